@@ -1,0 +1,203 @@
+// Auxiliary kernels: the scalar cross-check kernel, the split merge, dtype conversion.
+#include "attn_params.h"
+
+#include <hip/hip_fp16.h>
+
+namespace dg {
+
+namespace {
+
+template <typename T>
+__device__ __forceinline__ float load_elem(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float load_elem<uint16_t>(const uint16_t* p, int64_t i) {  // bf16 bits
+  return bf16_bits_to_f32(p[i]);
+}
+template <>
+__device__ __forceinline__ float load_elem<_Float16>(const _Float16* p, int64_t i) {
+  return (float)p[i];
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ void store_out(const AttnParams& p, size_t idx, float y) {
+  if (p.out_dtype == DT_F32) {
+    ((float*)p.out)[idx] = y;
+  } else if (p.out_dtype == DT_BF16) {
+    ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(y, p.out_trunc != 0);
+  } else {
+    ((_Float16*)p.out)[idx] = (_Float16)y;
+  }
+}
+
+// One wave per (canvas row, query head); keys streamed one at a time with the online
+// softmax recurrence.  Slow on purpose: it shares nothing with the MFMA kernel except the
+// mask arithmetic, which is what makes it a useful on-device cross-check.
+template <typename KT>
+__global__ void __launch_bounds__(64) attn_scalar_kernel(const AttnParams p, const uint32_t hd) {
+  const uint32_t tok = blockIdx.x, qh = blockIdx.y, lane = threadIdx.x;
+  const uint32_t kvh = qh / p.group;
+  const RowBounds b = row_bounds(p, tok);
+  const KT* kbase = (const KT*)p.k + (int64_t)kvh * p.k_head_stride;
+  const KT* vbase = (const KT*)p.v + (int64_t)kvh * p.v_head_stride;
+  const size_t qoff = ((size_t)tok * p.hq + qh) * hd;
+  float qv[8], acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t d = lane + 64u * i;
+    acc[i] = 0.f;
+    qv[i] = 0.f;
+    if (d < hd) {
+      qv[i] = p.q_is_bf16 ? bf16_bits_to_f32(((const uint16_t*)p.q)[qoff + d])
+                          : load_elem<KT>((const KT*)p.q, (int64_t)(qoff + d));
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  for (uint32_t t = b.lo; t < p.t_all; ++t) {
+    if (!key_visible(b, t, p.t_all)) {
+      if (t >= b.hi && b.extra >= p.t_all) break;
+      continue;
+    }
+    const int64_t slot = kv_slot(p.ring_mask, t);
+    const KT* kk = kbase + slot * p.k_tok_stride;
+    const KT* vv = vbase + slot * p.v_tok_stride;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t d = lane + 64u * i;
+      if (d < hd) s += qv[i] * load_elem<KT>(kk, d);
+    }
+    s = wave_sum(s) * p.scale_log2;
+    const float mn = fmaxf(m, s);
+    const float corr = exp2f(m - mn);
+    const float pr = exp2f(s - mn);
+    l = l * corr + pr;
+    m = mn;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t d = lane + 64u * i;
+      if (d < hd) acc[i] = acc[i] * corr + pr * load_elem<KT>(vv, d);
+    }
+  }
+  if (lane == 0) {
+    if (!(l > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l));
+    if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l > 0.f ? m * kLn2 + logf(l) : -INFINITY;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t d = lane + 64u * i;
+    if (d < hd) store_out(p, qoff + d, l > 0.f ? acc[i] / l : 0.f);
+  }
+}
+
+// One wave per stacked row: combines the per-split (m, l, O) triples.
+__global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, const uint32_t hd) {
+  const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t gr = blockIdx.x * 4 + wave;  // global stacked row over all KV heads
+  if (gr >= p.hkv * p.rows_total) return;
+  const uint32_t kvh = gr / p.rows_total, r = gr % p.rows_total;
+  const uint32_t tok = r / p.group, qh = kvh * p.group + r % p.group;
+  const size_t split_stride = (size_t)p.hkv * p.rows_pad;
+  const size_t row = (size_t)kvh * p.rows_pad + r;
+  float mx = -INFINITY;
+  for (uint32_t s = 0; s < p.n_splits; ++s) mx = fmaxf(mx, p.part_ml[(s * split_stride + row) * 2]);
+  float den = 0.f;
+  for (uint32_t s = 0; s < p.n_splits; ++s) {
+    const float ms = p.part_ml[(s * split_stride + row) * 2], ls = p.part_ml[(s * split_stride + row) * 2 + 1];
+    if (ls > 0.f) den += ls * exp2f(ms - mx);
+  }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  const size_t ooff = ((size_t)tok * p.hq + qh) * hd;
+  for (uint32_t d4 = lane; d4 < hd / 4; d4 += 64) {
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t s = 0; s < p.n_splits; ++s) {
+      const float ms = p.part_ml[(s * split_stride + row) * 2], ls = p.part_ml[(s * split_stride + row) * 2 + 1];
+      if (!(ls > 0.f)) continue;
+      const float w = exp2f(ms - mx);
+      const float4 a = ((const float4*)(p.part_o + (s * split_stride + row) * hd))[d4];
+      o.x += w * a.x;
+      o.y += w * a.y;
+      o.z += w * a.z;
+      o.w += w * a.w;
+    }
+    store_out(p, ooff + d4 * 4 + 0, o.x * inv);
+    store_out(p, ooff + d4 * 4 + 1, o.y * inv);
+    store_out(p, ooff + d4 * 4 + 2, o.z * inv);
+    store_out(p, ooff + d4 * 4 + 3, o.w * inv);
+  }
+  if (lane == 0) {
+    if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));
+    if (p.lse) p.lse[(size_t)tok * p.hq + qh] = den > 0.f ? mx * kLn2 + logf(den) : -INFINITY;
+  }
+}
+
+__device__ __forceinline__ float load_any(const void* src, uint32_t dt, size_t i) {
+  if (dt == DT_F32) return ((const float*)src)[i];
+  if (dt == DT_BF16) return bf16_bits_to_f32(((const uint16_t*)src)[i]);
+  return (float)((const _Float16*)src)[i];
+}
+__device__ __forceinline__ void store_any(void* dst, uint32_t dt, size_t i, float v) {
+  if (dt == DT_F32) ((float*)dst)[i] = v;
+  else if (dt == DT_BF16) ((uint16_t*)dst)[i] = f32_to_bf16_bits(v, false);
+  else ((_Float16*)dst)[i] = (_Float16)v;
+}
+
+__global__ void convert_kernel(const void* src, uint32_t sdt, void* dst, uint32_t ddt, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    store_any(dst, ddt, i, load_any(src, sdt, i));
+}
+
+__global__ void kv_gather_kernel(const void* src, uint32_t sdt, void* dst, uint32_t ddt, uint32_t hkv,
+                                 uint32_t t_all, uint32_t hd, int64_t tok_stride, int64_t head_stride,
+                                 uint32_t ring_mask) {
+  const size_t n = (size_t)hkv * t_all * hd;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const uint32_t d = (uint32_t)(i % hd);
+    const uint32_t t = (uint32_t)((i / hd) % t_all);
+    const uint32_t h = (uint32_t)(i / ((size_t)hd * t_all));
+    const int64_t s = (int64_t)kv_slot(ring_mask, t) * tok_stride + (int64_t)h * head_stride + d;
+    store_any(dst, ddt, i, load_any(src, sdt, (size_t)s));
+  }
+}
+
+}  // namespace
+
+hipError_t launch_attn_scalar(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s) {
+  dim3 grid(p.canvas, p.hq, 1), block(64, 1, 1);
+  if (kv_dtype == DT_BF16)
+    hipLaunchKernelGGL(attn_scalar_kernel<uint16_t>, grid, block, 0, s, p, head_dim);
+  else
+    hipLaunchKernelGGL(attn_scalar_kernel<_Float16>, grid, block, 0, s, p, head_dim);
+  return hipGetLastError();
+}
+
+hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, hipStream_t s) {
+  const uint32_t rows = p.hkv * p.rows_total;
+  hipLaunchKernelGGL(attn_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, p, head_dim);
+  return hipGetLastError();
+}
+
+hipError_t launch_convert(const void* src, uint32_t sdt, void* dst, uint32_t ddt, size_t n, hipStream_t s) {
+  if (n == 0) return hipSuccess;
+  const size_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(convert_kernel, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, src, sdt, dst,
+                     ddt, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_gather(const void* src, uint32_t sdt, void* dst, uint32_t ddt, uint32_t hkv, uint32_t t_all,
+                            uint32_t hd, int64_t tok_stride, int64_t head_stride, uint32_t ring_mask,
+                            hipStream_t s) {
+  const size_t n = (size_t)hkv * t_all * hd;
+  if (n == 0) return hipSuccess;
+  const size_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(kv_gather_kernel, dim3((unsigned)(blocks > 8192 ? 8192 : blocks)), dim3(256), 0, s, src, sdt, dst,
+                     ddt, hkv, t_all, hd, tok_stride, head_stride, ring_mask);
+  return hipGetLastError();
+}
+
+}  // namespace dg

@@ -1,0 +1,105 @@
+// Kernel-side argument block and mask arithmetic shared by every attention kernel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dg {
+
+enum : uint32_t { DT_BF16 = 0, DT_F16 = 1, DT_F32 = 2 };
+
+constexpr int kBlockM = 128;   // stacked query rows per workgroup (4 waves x 32)
+constexpr int kBlockN = 32;    // keys per tile
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Stacked row r of a KV head = tok * group + g: the `group` query heads that share one KV
+// head sit next to each other, so a 128-row tile covers 128/group consecutive canvas rows.
+struct AttnParams {
+  const void* q;       // [canvas][hq][D], element type = KV element type unless q_is_bf16
+  const void* k;       // layer region + K offset (element type E)
+  const void* v;       // layer region + V offset
+  void* out;           // [canvas][hq][D]
+  float* lse;          // [canvas][hq] or null
+  float* part_o;       // [split][hkv][rows_pad][D] unnormalised accumulators
+  float* part_ml;      // [split][hkv][rows_pad][2] (m in log2 units, l)
+  uint32_t* dbg;       // 4 words, first-writer-wins, or null
+  int64_t k_tok_stride, k_head_stride, v_tok_stride, v_head_stride;  // elements
+  uint32_t canvas, hq, hkv, group;
+  uint32_t kv_len, t_all;
+  uint32_t causal_rows;
+  uint32_t win_m1;       // window-1, or 0xffffffff when unwindowed
+  uint32_t lo_nc;        // first visible key of a non-causal row
+  uint32_t extra_lo;     // causal rows also see keys >= extra_lo (t_all = none)
+  uint32_t ring_mask;
+  uint32_t rows_total, rows_pad, n_mtiles;
+  uint32_t n_splits, tile_first, tiles_per_split, tile_end;
+  uint32_t q_is_bf16;    // Q holds bf16 although E is f16 (reference: bf16 activations, f16 cache)
+  uint32_t out_dtype, out_trunc;
+  float scale_log2;      // softmax_scale * log2(e)
+};
+
+struct RowBounds {
+  uint32_t lo, hi, extra;  // visible iff (lo <= t < hi) or (extra <= t), and t < t_all
+};
+
+// Reference rules: causal rows see [max(0,qpos-(window-1)), qpos]; the other rows see
+// [lo_nc, t_all) where lo_nc = max(0, kv_len-(window-1)) unless the caller set it.
+__device__ __forceinline__ RowBounds row_bounds(const AttnParams& p, uint32_t tok) {
+  RowBounds b;
+  const bool causal = tok < p.causal_rows;
+  const uint32_t qpos = p.kv_len + tok;
+  if (causal) {
+    b.hi = min(p.t_all, qpos + 1u);
+    b.lo = (p.win_m1 != 0xffffffffu && qpos > p.win_m1) ? qpos - p.win_m1 : 0u;
+    b.extra = p.extra_lo;
+  } else {
+    b.hi = p.t_all;
+    b.lo = p.lo_nc;
+    b.extra = p.t_all;
+  }
+  return b;
+}
+
+__device__ __forceinline__ bool key_visible(const RowBounds& b, uint32_t t, uint32_t t_all) {
+  return t < t_all && ((t >= b.lo && t < b.hi) || t >= b.extra);
+}
+
+__device__ __forceinline__ uint32_t kv_slot(uint32_t ring_mask, uint32_t t) {
+  return ring_mask ? (t & ring_mask) : t;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+  return __uint_as_float((uint32_t)b << 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f, bool trunc) {
+  uint32_t u = __float_as_uint(f);
+  if (!trunc) {
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+  }
+  return (uint16_t)(u >> 16);
+}
+
+// first-writer-wins status record, like the reference's DebugStatus buffer
+__device__ __forceinline__ void dbg_report(uint32_t* dbg, uint32_t code, uint32_t tg, uint32_t value) {
+  if (dbg == nullptr) return;
+  if (atomicCAS(dbg, 0u, code) == 0u) {
+    dbg[1] = 7u;
+    dbg[2] = tg;
+    dbg[3] = value;
+  }
+}
+
+// host-side launchers (defined next to their kernels)
+hipError_t launch_attn_scalar(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
+hipError_t launch_attn_mfma(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
+hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, hipStream_t s);
+hipError_t launch_convert(const void* src, uint32_t src_dtype, void* dst, uint32_t dst_dtype, size_t n, hipStream_t s);
+// gathers keys [0,t_all) of a strided (possibly ring) cache into planes [hkv][t_all][D] of dst_dtype
+hipError_t launch_kv_gather(const void* src, uint32_t src_dtype, void* dst, uint32_t dst_dtype, uint32_t hkv,
+                            uint32_t t_all, uint32_t head_dim, int64_t tok_stride, int64_t head_stride,
+                            uint32_t ring_mask, hipStream_t s);
+
+}  // namespace dg

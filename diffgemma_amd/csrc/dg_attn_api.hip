@@ -1,0 +1,392 @@
+// extern "C" boundary of libdg_attn_hip.so: descriptor validation, launch planning, and the
+// reference-shaped dispatch entry.  No allocation, no host synchronisation, no exceptions.
+#include "../../include/dg_attn.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+
+#include "attn_params.h"
+
+namespace {
+
+constexpr uint32_t kMaxSplits = 64;
+constexpr size_t kAlign = 256;
+
+inline size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
+inline uint32_t elem_size(uint32_t dt) { return dt == DG_F32 ? 4u : 2u; }
+inline bool is_pow2(uint64_t x) { return x && !(x & (x - 1)); }
+
+struct DeviceInfo {
+  int checked = 0;  // 0 unknown, 1 ok, -1 wrong arch
+  int cus = 256;
+};
+DeviceInfo g_dev[64];
+thread_local uint32_t* g_tls_dbg = nullptr;
+std::mutex g_dev_mu;
+
+int device_info(DeviceInfo* out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DG_ERR_DEVICE;
+  std::lock_guard<std::mutex> lock(g_dev_mu);
+  DeviceInfo& di = g_dev[dev];
+  if (di.checked == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return DG_ERR_DEVICE;
+    di.checked = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    di.cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  if (di.checked < 0) return DG_ERR_DEVICE;
+  *out = di;
+  return DG_OK;
+}
+
+// Everything the launch needs that can be derived on the host without a device.
+struct Plan {
+  uint32_t group = 0, rows_total = 0, n_mtiles = 0, rows_pad = 0;
+  uint32_t t_all = 0, lo_nc = 0, extra_lo = 0, win_m1 = 0xffffffffu;
+  uint32_t tile_first = 0, tile_end = 0, tiles_per_split = 0, n_splits = 1;
+  uint32_t e_dtype = DG_BF16;   // element type the kernels compute in (bf16 or f16)
+  bool convert_q = false, gather_kv = false, q_is_bf16 = false;
+  bool scalar = false;
+  size_t off_q = 0, off_kv = 0, off_part_o = 0, off_part_ml = 0, total = 0;
+  float scale = 1.0f;
+};
+
+int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
+  if (!d) return DG_ERR_NULL;
+  const uint32_t hd = d->head_dim;
+  if (d->canvas == 0 || d->canvas > 65536 || d->n_q_heads == 0 || d->n_kv_heads == 0) return DG_ERR_SHAPE;
+  if (d->n_q_heads % d->n_kv_heads != 0 || d->n_q_heads > 65535) return DG_ERR_SHAPE;
+  if (d->kernel > DG_KERNEL_MFMA) return DG_ERR_UNSUPPORTED;
+  pl->scalar = d->kernel == DG_KERNEL_SCALAR;
+  if (pl->scalar) {
+    if (hd == 0 || hd > 512 || hd % 8 != 0) return DG_ERR_SHAPE;
+  } else if (hd != 32 && hd != 64 && hd != 128 && hd != 256 && hd != 512) {
+    return DG_ERR_SHAPE;
+  }
+  if ((uint64_t)d->kv_len + d->canvas > 0x7fffffffull) return DG_ERR_SHAPE;
+  if (d->q_dtype > DG_F32 || d->kv_dtype > DG_F32 || d->out_dtype > DG_F32) return DG_ERR_DTYPE;
+  if (d->out_dtype == DG_F16) return DG_ERR_DTYPE;
+  if (d->causal_rows > d->canvas) return DG_ERR_MASK;
+  if (d->kv_ring_mask != 0) {
+    if (!is_pow2((uint64_t)d->kv_ring_mask + 1) || d->kv_ring_mask + 1 < (uint32_t)dg::kBlockN) return DG_ERR_LAYOUT;
+  }
+  pl->t_all = d->kv_len + d->canvas;
+  if ((d->flags & DG_ATTN_F_T_LO_EXPLICIT) && d->t_lo > pl->t_all) return DG_ERR_MASK;
+  if (!(d->softmax_scale >= 0.0f)) return DG_ERR_MASK;
+  pl->scale = d->softmax_scale == 0.0f ? 1.0f : d->softmax_scale;
+
+  // element type: the cache decides; f32 anywhere is brought down to f16 first
+  pl->e_dtype = d->kv_dtype == DG_BF16 ? DG_BF16 : DG_F16;
+  pl->gather_kv = d->kv_dtype == DG_F32;
+  if (d->q_dtype == DG_F32) {
+    pl->convert_q = true;
+  } else if (d->q_dtype == DG_BF16 && pl->e_dtype == DG_F16) {
+    pl->q_is_bf16 = true;  // bf16 activations over an f16 cache: the reference's own pairing
+  } else if (d->q_dtype != pl->e_dtype) {
+    return DG_ERR_DTYPE;   // f16 Q over a bf16 cache
+  }
+
+  if (!pl->gather_kv) {
+    // rows must be 16-byte addressable for the direct-to-LDS loads
+    const int64_t s[5] = {d->k_tok_stride, d->k_head_stride, d->v_base_off, d->v_tok_stride, d->v_head_stride};
+    for (int64_t x : s)
+      if (x < 0 || x % 8 != 0) return DG_ERR_LAYOUT;
+    if (d->kv_region_bytes % 16 != 0) return DG_ERR_LAYOUT;
+    if (d->k_tok_stride < (int64_t)hd || d->v_tok_stride < (int64_t)hd) return DG_ERR_LAYOUT;
+    if (d->k_tok_stride * 2 * dg::kBlockN >= (1ll << 31) || d->v_tok_stride * 2 * dg::kBlockN >= (1ll << 31))
+      return DG_ERR_LAYOUT;
+  } else {
+    if (d->k_tok_stride < 0 || d->k_head_stride < 0 || d->v_base_off < 0 || d->v_tok_stride < 0 ||
+        d->v_head_stride < 0)
+      return DG_ERR_LAYOUT;
+  }
+
+  pl->group = d->n_q_heads / d->n_kv_heads;
+  pl->rows_total = d->canvas * pl->group;
+  pl->n_mtiles = (pl->rows_total + dg::kBlockM - 1) / dg::kBlockM;
+  pl->rows_pad = pl->n_mtiles * dg::kBlockM;
+
+  // mask constants (reference rules, src/shaders/attn/attention/attention.metal:49-63)
+  pl->win_m1 = d->window ? d->window - 1u : 0xffffffffu;
+  pl->lo_nc = (d->window && d->kv_len > d->window - 1u) ? d->kv_len - (d->window - 1u) : 0u;
+  if (d->flags & DG_ATTN_F_T_LO_EXPLICIT) pl->lo_nc = d->t_lo;
+  pl->extra_lo = (d->flags & DG_ATTN_F_CAUSAL_SEES_MASKED) ? std::min(d->kv_len + d->causal_rows, pl->t_all) : pl->t_all;
+
+  // key tiles any row can see
+  uint32_t lo_all = 0xffffffffu;
+  if (d->causal_rows < d->canvas) lo_all = std::min(lo_all, pl->lo_nc);
+  if (d->causal_rows > 0) {
+    const uint32_t qpos0 = d->kv_len;
+    lo_all = std::min(lo_all, (d->window && qpos0 > d->window - 1u) ? qpos0 - (d->window - 1u) : 0u);
+  }
+  lo_all = std::min(lo_all, pl->t_all);
+  pl->tile_first = lo_all / dg::kBlockN;
+  pl->tile_end = (pl->t_all + dg::kBlockN - 1) / dg::kBlockN;
+  const uint32_t ntiles = std::max(1u, pl->tile_end - pl->tile_first);
+
+  uint32_t splits = d->n_splits;
+  if (pl->scalar) {
+    splits = 1;
+  } else if (splits == 0) {
+    // enough workgroups for every CU, but no split shorter than 4 tiles
+    const uint32_t base = d->n_kv_heads * pl->n_mtiles;
+    splits = std::max(1u, (uint32_t)cus / std::max(1u, base));
+    splits = std::min(splits, std::max(1u, ntiles / 4u));
+  }
+  splits = std::min(std::min(splits, kMaxSplits), ntiles);
+  pl->tiles_per_split = (ntiles + splits - 1) / splits;
+  pl->n_splits = (ntiles + pl->tiles_per_split - 1) / pl->tiles_per_split;
+
+  // workspace carve-up
+  size_t off = 0;
+  if (pl->convert_q) {
+    pl->off_q = off;
+    off += align_up((size_t)d->canvas * d->n_q_heads * hd * 2);
+  }
+  if (pl->gather_kv) {
+    pl->off_kv = off;
+    off += align_up((size_t)2 * d->n_kv_heads * pl->t_all * hd * 2);
+  }
+  if (pl->n_splits > 1) {
+    pl->off_part_o = off;
+    off += align_up((size_t)pl->n_splits * d->n_kv_heads * pl->rows_pad * hd * 4);
+    pl->off_part_ml = off;
+    off += align_up((size_t)pl->n_splits * d->n_kv_heads * pl->rows_pad * 2 * 4);
+  }
+  pl->total = off;
+  return DG_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint32_t dg_attn_abi_version(void) { return DG_ATTN_ABI_VERSION; }
+
+const char* dg_attn_strerror(int status) {
+  switch (status) {
+    case DG_OK: return "ok";
+    case DG_ERR_NULL: return "required pointer is null";
+    case DG_ERR_SHAPE: return "unsupported canvas / head count / head_dim";
+    case DG_ERR_DTYPE: return "unsupported dtype tag or dtype combination";
+    case DG_ERR_LAYOUT: return "KV strides or offsets not usable (16-byte alignment, ring mask, range)";
+    case DG_ERR_WORKSPACE: return "workspace missing or too small";
+    case DG_ERR_MASK: return "inconsistent mask description";
+    case DG_ERR_LAUNCH: return "HIP launch failed";
+    case DG_ERR_DEVICE: return "no gfx950 device current";
+    case DG_ERR_UNSUPPORTED: return "request not implemented";
+    default: return "unknown status";
+  }
+}
+
+void dg_attn_desc_reference_layout(dg_attn_desc* d) {
+  const int64_t row = (int64_t)d->n_kv_heads * d->head_dim;
+  d->k_tok_stride = 2 * row;
+  d->k_head_stride = d->head_dim;
+  d->v_base_off = row;
+  d->v_tok_stride = 2 * row;
+  d->v_head_stride = d->head_dim;
+}
+
+void dg_attn_desc_head_major_layout(dg_attn_desc* d, uint64_t t_cap) {
+  d->k_tok_stride = d->head_dim;
+  d->k_head_stride = (int64_t)t_cap * d->head_dim;
+  d->v_base_off = (int64_t)d->n_kv_heads * (int64_t)t_cap * d->head_dim;
+  d->v_tok_stride = d->head_dim;
+  d->v_head_stride = (int64_t)t_cap * d->head_dim;
+}
+
+int dg_attn_workspace_bytes(const dg_attn_desc* d, size_t* out_bytes) {
+  if (!d || !out_bytes) return DG_ERR_NULL;
+  Plan pl;
+  // Sized for a 256-CU part whatever device is current, so the answer does not depend on it.
+  const int rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  *out_bytes = pl.total;
+  return DG_OK;
+}
+
+int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits) {
+  if (!d || !out_splits) return DG_ERR_NULL;
+  Plan pl;
+  const int rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  *out_splits = pl.n_splits;
+  return DG_OK;
+}
+
+int dg_attn_visible_pairs(const dg_attn_desc* d, uint64_t* pairs, double* flops) {
+  if (!d) return DG_ERR_NULL;
+  Plan pl;
+  const int rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  uint64_t n = 0;
+  for (uint32_t tok = 0; tok < d->canvas; ++tok) {
+    const bool causal = tok < d->causal_rows;
+    const uint32_t qpos = d->kv_len + tok;
+    uint32_t lo, hi, extra;
+    if (causal) {
+      hi = std::min(pl.t_all, qpos + 1u);
+      lo = (d->window && qpos > d->window - 1u) ? qpos - (d->window - 1u) : 0u;
+      extra = pl.extra_lo;
+    } else {
+      hi = pl.t_all;
+      lo = pl.lo_nc;
+      extra = pl.t_all;
+    }
+    if (hi > lo) n += hi - lo;
+    const uint32_t e = std::max(extra, std::max(hi, lo));
+    if (pl.t_all > e) n += pl.t_all - e;
+  }
+  if (pairs) *pairs = n;
+  if (flops) *flops = 4.0 * d->head_dim * d->n_q_heads * (double)n;
+  return DG_OK;
+}
+
+int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  if (pl.total > 0 && (!workspace || workspace_bytes < pl.total)) return DG_ERR_WORKSPACE;
+  if (pl.total > 0 && ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
+  if (((uintptr_t)q % 16) != 0 || ((uintptr_t)kv_base % 16) != 0 || ((uintptr_t)out % 16) != 0) return DG_ERR_LAYOUT;
+  hipStream_t s = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  const uint32_t hd = d->head_dim;
+  const uint32_t esz_kv = elem_size(d->kv_dtype);
+
+  dg::AttnParams p;
+  std::memset(&p, 0, sizeof(p));
+  const char* region = (const char*)kv_base + d->kv_region_bytes;
+  p.q = q;
+  p.ring_mask = d->kv_ring_mask;
+  if (pl.convert_q) {
+    if (dg::launch_convert(q, d->q_dtype, ws + pl.off_q, pl.e_dtype, (size_t)d->canvas * d->n_q_heads * hd, s) != hipSuccess)
+      return DG_ERR_LAUNCH;
+    p.q = ws + pl.off_q;
+  }
+  if (pl.gather_kv) {
+    char* kp = ws + pl.off_kv;
+    char* vp = kp + (size_t)d->n_kv_heads * pl.t_all * hd * 2;
+    if (dg::launch_kv_gather(region, d->kv_dtype, kp, pl.e_dtype, d->n_kv_heads, pl.t_all, hd, d->k_tok_stride,
+                             d->k_head_stride, d->kv_ring_mask, s) != hipSuccess)
+      return DG_ERR_LAUNCH;
+    if (dg::launch_kv_gather(region + d->v_base_off * (int64_t)esz_kv, d->kv_dtype, vp, pl.e_dtype, d->n_kv_heads,
+                             pl.t_all, hd, d->v_tok_stride, d->v_head_stride, d->kv_ring_mask, s) != hipSuccess)
+      return DG_ERR_LAUNCH;
+    p.k = kp;
+    p.v = vp;
+    p.k_tok_stride = p.v_tok_stride = hd;
+    p.k_head_stride = p.v_head_stride = (int64_t)pl.t_all * hd;
+    p.ring_mask = 0;
+  } else {
+    p.k = region;
+    p.v = region + d->v_base_off * 2;
+    p.k_tok_stride = d->k_tok_stride;
+    p.k_head_stride = d->k_head_stride;
+    p.v_tok_stride = d->v_tok_stride;
+    p.v_head_stride = d->v_head_stride;
+  }
+  p.out = out;
+  p.lse = lse;
+  p.dbg = nullptr;
+  p.canvas = d->canvas;
+  p.hq = d->n_q_heads;
+  p.hkv = d->n_kv_heads;
+  p.group = pl.group;
+  p.kv_len = d->kv_len;
+  p.t_all = pl.t_all;
+  p.causal_rows = d->causal_rows;
+  p.win_m1 = pl.win_m1;
+  p.lo_nc = pl.lo_nc;
+  p.extra_lo = pl.extra_lo;
+  p.rows_total = pl.rows_total;
+  p.rows_pad = pl.rows_pad;
+  p.n_mtiles = pl.n_mtiles;
+  p.n_splits = pl.n_splits;
+  p.tile_first = pl.tile_first;
+  p.tiles_per_split = pl.tiles_per_split;
+  p.tile_end = pl.tile_end;
+  p.q_is_bf16 = pl.q_is_bf16 ? 1u : 0u;
+  p.out_dtype = d->out_dtype;
+  p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
+  p.scale_log2 = pl.scale * dg::kLog2e;
+  if (pl.n_splits > 1) {
+    p.part_o = (float*)(ws + pl.off_part_o);
+    p.part_ml = (float*)(ws + pl.off_part_ml);
+  }
+  p.dbg = g_tls_dbg;  // set only while dg_attention_dispatch is on the stack
+
+  if (pl.scalar) {
+    if (dg::launch_attn_scalar(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+    return DG_OK;
+  }
+  if (dg::launch_attn_mfma(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+  if (pl.n_splits > 1 && dg::launch_attn_merge(p, hd, s) != hipSuccess) return DG_ERR_LAUNCH;
+  return DG_OK;
+}
+
+static void desc_from_reference(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                                dg_attn_desc* d) {
+  std::memset(d, 0, sizeof(*d));
+  d->canvas = dims->canvas;
+  d->n_q_heads = dims->n_q_heads;
+  d->n_kv_heads = L->n_kv_heads;
+  d->head_dim = L->head_dim;
+  d->kv_len = kv_len;
+  d->causal_rows = dims->causal ? dims->canvas : 0u;
+  d->window = dims->window;
+  d->kv_ring_mask = L->kv_ring_mask;
+  d->q_dtype = DG_BF16;
+  d->kv_dtype = DG_F16;
+  d->out_dtype = DG_BF16;
+  d->flags = DG_ATTN_F_OUT_TRUNCATE;
+  d->kv_region_bytes = L->kv_region;
+  dg_attn_desc_reference_layout(d);
+}
+
+int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                             size_t* out_bytes) {
+  if (!L || !dims || !out_bytes) return DG_ERR_NULL;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, kv_len, &d);
+  return dg_attn_workspace_bytes(&d, out_bytes);
+}
+
+int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                          const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg,
+                          void* attn_state, size_t attn_state_bytes, void* stream) {
+  if (!L || !P || !dims) return DG_ERR_NULL;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, P->kv_len, &d);
+  g_tls_dbg = (uint32_t*)dbg;
+  const int rc = dg_attn_forward(&d, q, kvcache, out, nullptr, attn_state, attn_state_bytes, stream);
+  g_tls_dbg = nullptr;
+  return rc;
+}
+
+uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype) { return (uint64_t)head_dim * elem_size(kv_dtype); }
+
+uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slots, uint32_t kv_dtype) {
+  return slots * (uint64_t)n_kv_heads * 2ull * dg_kv_row_bytes(head_dim, kv_dtype);
+}
+
+uint64_t dg_kv_slot(uint32_t kv_ring_mask, uint64_t pos) { return kv_ring_mask ? (pos & kv_ring_mask) : pos; }
+
+uint64_t dg_layer_kv_slots(int is_full, uint64_t max_seq, uint64_t ring_slots_cap) {
+  if (is_full) return (max_seq + 8 + 7) / 8 * 8;
+  uint64_t p2 = 1;
+  while (p2 < max_seq) p2 <<= 1;
+  return ring_slots_cap ? std::min(p2, ring_slots_cap) : p2;
+}
+
+}  // extern "C"

@@ -1,0 +1,171 @@
+/* C-ABI of the MI355X (gfx950) denoise-step attention library, libdg_attn_hip.so.
+ *
+ * Every entry point takes plain pointers and sizes: device pointers are caller-owned HIP
+ * allocations, `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ * Calls enqueue work in order on that stream, never synchronise the host, never allocate,
+ * and never unwind across the boundary; 0 means success, a negative value is a dg_status
+ * (dg_attn_strerror gives the text).  One thread drives one stream, as in the reference
+ * ("one thread owns the GPU + KV", reference ARCHITECTURE.md:553).
+ *
+ * Reference interfaces replaced (paths relative to the reference root):
+ *   dg_attention_dispatch    StepEnc::encode_layer_attention_dispatch,
+ *                            src/metal/step_kernel/enc.rs:2102-2296 (buffers 0..8 it binds)
+ *   dg_attn_forward          the kernels behind it: attention, attention_mma2, attention_mma_full
+ *                            (src/shaders/attn/attention/ *.metal files) and their harnesses
+ *                            attention::gpu / gpu_mma2 / gpu_mma_full (attention/mod.rs:377-686)
+ *   dg_layer_offsets         LayerOffsets, src/metal/step_kernel/mod.rs:132-167
+ *   dg_step_params           StepParams,   src/metal/step_kernel/mod.rs:189-213
+ *   dg_attn_dims             AttnDims,     src/shaders/attn/qk_rope_kv/mod.rs:15-38
+ *   dg_attn_block_range      AttnBlockRange, src/shaders/include/attention_device.metal:160-165
+ *   dg_debug_status          DebugStatus,  src/metal/debug_status.rs:11-43
+ *   dg_kv_*                  kv_row_bytes / kv_region_bytes / kv_slot / layer_kv_slots,
+ *                            src/metal/step_kv/mod.rs:65-100, src/metal/step_kernel/mod.rs:511-527
+ */
+#ifndef DG_ATTN_H
+#define DG_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DG_ATTN_ABI_VERSION 1u
+
+typedef enum dg_status {
+  DG_OK = 0,
+  DG_ERR_NULL = -1,        /* a required pointer is NULL */
+  DG_ERR_SHAPE = -2,       /* canvas/head counts/head_dim not supported */
+  DG_ERR_DTYPE = -3,       /* dtype tag or dtype combination not supported */
+  DG_ERR_LAYOUT = -4,      /* strides / offsets not 16-byte aligned, ring mask not 2^k-1, ... */
+  DG_ERR_WORKSPACE = -5,   /* workspace missing or too small */
+  DG_ERR_MASK = -6,        /* causal_rows > canvas, window/t_lo inconsistent */
+  DG_ERR_LAUNCH = -7,      /* the HIP runtime refused a launch (sticky error text kept) */
+  DG_ERR_DEVICE = -8,      /* not a gfx950 device, or no device */
+  DG_ERR_UNSUPPORTED = -9  /* valid request the library does not implement (e.g. q8 KV) */
+} dg_status;
+
+typedef enum dg_dtype { DG_BF16 = 0, DG_F16 = 1, DG_F32 = 2 } dg_dtype;
+
+typedef enum dg_kernel_sel {
+  DG_KERNEL_AUTO = 0,   /* MFMA kernel, split count chosen by the library */
+  DG_KERNEL_SCALAR = 1, /* one wave per (row, head): the slow on-GPU cross-check, like the
+                           reference's scalar `attention` kernel next to its MMA kernels */
+  DG_KERNEL_MFMA = 2
+} dg_kernel_sel;
+
+/* desc.flags */
+#define DG_ATTN_F_OUT_TRUNCATE 0x1u        /* bf16/f16 store by truncation (reference arena_store,
+                                              src/shaders/include/common.metal:16-18); default RNE */
+#define DG_ATTN_F_CAUSAL_SEES_MASKED 0x2u  /* causal rows also see canvas keys >= kv_len+causal_rows */
+#define DG_ATTN_F_T_LO_EXPLICIT 0x4u       /* non-causal rows start at desc.t_lo instead of the
+                                              window rule kv_len-(window-1) */
+
+typedef struct dg_attn_desc {
+  uint32_t canvas;        /* query rows; the reference passes active_canvas (256/128/64) */
+  uint32_t n_q_heads;
+  uint32_t n_kv_heads;
+  uint32_t head_dim;      /* 32, 64, 128, 256 or 512 */
+  uint32_t kv_len;        /* committed prefix length; canvas keys live at [kv_len, kv_len+canvas) */
+  uint32_t causal_rows;   /* 0 = denoise (reference causal=0); canvas = reference causal=1;
+                             in between = rows below it causal, rows from it on bidirectional */
+  uint32_t window;        /* 0 = global layer; else reference rule: non-causal rows see keys
+                             >= kv_len-(window-1), causal row at qpos sees >= qpos-(window-1) */
+  uint32_t kv_ring_mask;  /* 0 = linear; else slot = pos & mask (mask+1 a power of two) */
+  uint32_t q_dtype;       /* dg_dtype: DG_BF16 or DG_F32 */
+  uint32_t kv_dtype;      /* dg_dtype: DG_BF16, DG_F16 or DG_F32 */
+  uint32_t out_dtype;     /* dg_dtype: DG_BF16 or DG_F32 */
+  uint32_t flags;
+  uint32_t t_lo;          /* used with DG_ATTN_F_T_LO_EXPLICIT */
+  uint32_t n_splits;      /* key-range splits; 0 = library chooses */
+  uint32_t kernel;        /* dg_kernel_sel */
+  float    softmax_scale; /* multiplies q.k; 0 means 1.0 (the reference applies no scale) */
+  uint64_t kv_region_bytes; /* byte offset of this layer's region inside kv_base */
+  /* element strides/offsets inside the region (elements of kv_dtype), head_dim contiguous */
+  int64_t  k_tok_stride, k_head_stride;
+  int64_t  v_base_off, v_tok_stride, v_head_stride;
+} dg_attn_desc;
+
+/* Strides of the reference's slot-major cache [slot][K: Hkv*d | V: Hkv*d]
+ * (src/metal/step_kv/mod.rs:8-22). */
+void dg_attn_desc_reference_layout(dg_attn_desc* d);
+/* Strides of two planes [Hkv][t_cap][d] (K plane, then V plane at Hkv*t_cap*d). */
+void dg_attn_desc_head_major_layout(dg_attn_desc* d, uint64_t t_cap);
+
+/* Bytes of device scratch dg_attn_forward needs for this descriptor (0 is possible). */
+int dg_attn_workspace_bytes(const dg_attn_desc* d, size_t* out_bytes);
+
+/* Splits the library would use for this descriptor (n_splits==0 resolved). */
+int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits);
+
+/* q, out: [canvas][n_q_heads][head_dim]; lse: [canvas][n_q_heads] fp32 natural-log
+ * log-sum-exp of the scaled scores (NULL to skip; a row with no visible key gets -inf and
+ * an all-zero output row). */
+int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+const char* dg_attn_strerror(int status);
+uint32_t dg_attn_abi_version(void);
+/* Visible (row,key) pairs per head and the FLOP count 4*head_dim*n_q_heads*pairs
+ * (reference convention, src/commands/bench.rs:535-536). */
+int dg_attn_visible_pairs(const dg_attn_desc* d, uint64_t* pairs, double* flops);
+
+/* ---- the reference's own argument block, for a drop-in call site ---- */
+
+typedef struct dg_layer_offsets {
+  uint64_t input_ln, q_proj, q_norm, k_proj, k_norm, v_proj, o_proj, post_attn_ln;
+  uint64_t pre_ff_ln, mlp_gate, mlp_up, mlp_down, post_ff_ln_1;
+  uint64_t router_scale, router_proj, per_expert_scale, pre_ff_ln_2;
+  uint64_t experts_gate_up, experts_down, post_ff_ln_2, post_ff_ln, layer_scalar;
+  uint64_t kv_region;
+  uint32_t head_dim, n_kv_heads, is_full, kv_ring_mask;
+} dg_layer_offsets;
+
+typedef struct dg_step_params {
+  uint32_t kv_len, max_steps;
+  float entropy_bound, t_min, t_max, conf_threshold;
+  uint32_t stability_threshold, min_early_stop_steps, accept_plateau_threshold;
+  float plateau_prefix_mean_max;
+  uint32_t eos_token_id, kv_write_end;
+} dg_step_params;
+
+typedef struct dg_attn_dims {
+  uint32_t canvas, n_q_heads, causal, window;
+} dg_attn_dims;
+
+typedef struct dg_attn_block_range {
+  uint32_t t_begin, t_end, is_first, is_last;
+} dg_attn_block_range;
+
+typedef struct dg_debug_status {
+  uint32_t code, kernel_id, tg_id, value;
+} dg_debug_status;
+
+#define DG_DBG_ATTN_NONPOSITIVE_L 1u  /* a row's softmax denominator was not > 0 */
+#define DG_DBG_ATTN_NONFINITE_OUT 2u  /* an output element was NaN/inf */
+#define DG_DBG_KERNEL_ATTENTION 7u
+
+/* One layer's attention with exactly the buffers encode_layer_attention_dispatch binds:
+ * q = arena+attnq_off (bf16 [canvas][16][hd]), kvcache = whole KV buffer (f16, the kernel adds
+ * L->kv_region), out = arena+attno_off, L/P/dims are HOST structs (the reference binds L and P
+ * as device buffers; a host copy is what its encoder holds when it encodes the dispatch).
+ * dbg: device dg_debug_status (first-writer-wins) or NULL.  attn_state: device scratch of at
+ * least dg_attention_state_bytes() bytes (the reference's attn_state buffer, enc.rs:2214-2216).
+ * Output is stored with the reference's truncating bf16 store. */
+int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                          const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg,
+                          void* attn_state, size_t attn_state_bytes, void* stream);
+int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                             size_t* out_bytes);
+
+/* ---- KV-cache layout arithmetic (host) ---- */
+uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);
+uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slots, uint32_t kv_dtype);
+uint64_t dg_kv_slot(uint32_t kv_ring_mask, uint64_t pos);
+uint64_t dg_layer_kv_slots(int is_full, uint64_t max_seq, uint64_t ring_slots_cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,241 @@
+"""ctypes binding of the CPU oracle (libdg_attn_oracle.so).  TEST INFRASTRUCTURE ONLY.
+
+Imported by tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg — never by the
+diffgemma_amd package.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+ORACLE_DIR = Path(__file__).resolve().parent
+LIB_PATH = ORACLE_DIR / "libdg_attn_oracle.so"
+
+
+class Desc(C.Structure):
+    _fields_ = [
+        ("canvas", C.c_uint32), ("n_q_heads", C.c_uint32), ("n_kv_heads", C.c_uint32), ("head_dim", C.c_uint32),
+        ("kv_len", C.c_uint32), ("causal_rows", C.c_uint32), ("window", C.c_uint32), ("kv_ring_mask", C.c_uint32),
+        ("causal_sees_masked", C.c_uint32), ("strict_order", C.c_uint32),
+        ("t_lo_override", C.c_int64),
+        ("k_off", C.c_int64), ("k_tok_stride", C.c_int64), ("k_head_stride", C.c_int64),
+        ("v_off", C.c_int64), ("v_tok_stride", C.c_int64), ("v_head_stride", C.c_int64),
+        ("scale", C.c_float),
+    ]
+
+
+def build(force: bool = False) -> Path:
+    if force or not LIB_PATH.exists():
+        subprocess.run(["make", "-C", str(ORACLE_DIR), "-B" if force else "-s"], check=True,
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        build()
+    lib = C.CDLL(str(LIB_PATH))
+    P, VP = C.POINTER, C.c_void_p
+    lib.dgo_desc_reference_layout.argtypes = [P(Desc)]
+    lib.dgo_desc_head_major_layout.argtypes = [P(Desc), C.c_int64]
+    lib.dgo_visible.argtypes = [P(Desc), C.c_uint32, C.c_uint32]
+    lib.dgo_visible.restype = C.c_int
+    lib.dgo_visible_pairs.argtypes = [P(Desc)]
+    lib.dgo_visible_pairs.restype = C.c_uint64
+    lib.dgo_attention_f32.argtypes = [P(Desc), VP, VP, VP, VP, VP, C.c_uint32, C.c_int]
+    lib.dgo_attention_f64.argtypes = [P(Desc), VP, VP, VP, VP, VP, C.c_uint32, C.c_int]
+    lib.dgo_attention_blocked_f32.argtypes = [P(Desc), VP, VP, VP, VP, C.c_uint32, C.c_int]
+    lib.dgo_attention_partial_f32.argtypes = [P(Desc), VP, VP, C.c_uint32, C.c_uint32, VP, VP, VP, C.c_int]
+    lib.dgo_merge_partials_f32.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, VP, VP, VP, VP, VP]
+    lib.dgo_attention_bitmap_f32.argtypes = [C.c_uint32] * 5 + [VP] * 5
+    for name in ("dgo_f32_to_bf16_trunc", "dgo_f32_to_bf16_rne", "dgo_f32_to_f16_trunc", "dgo_f32_to_f16_rne"):
+        getattr(lib, name).argtypes = [C.c_float]
+        getattr(lib, name).restype = C.c_uint16
+    lib.dgo_bf16_to_f32.argtypes = [C.c_uint16]
+    lib.dgo_bf16_to_f32.restype = C.c_float
+    lib.dgo_f16_to_f32.argtypes = [C.c_uint16]
+    lib.dgo_f16_to_f32.restype = C.c_float
+    lib.dgo_round_array.argtypes = [VP, C.c_size_t, C.c_int]
+    lib.dgo_to_bits.argtypes = [VP, VP, C.c_size_t, C.c_int]
+    lib.dgo_from_bits.argtypes = [VP, VP, C.c_size_t, C.c_int]
+    lib.dgo_rms_norm_no_scale.argtypes = [VP, VP, C.c_size_t, C.c_float]
+    lib.dgo_rms_norm_head.argtypes = [VP, VP, C.c_size_t, C.c_float]
+    lib.dgo_fixture_tiny.argtypes = [VP, VP]
+    lib.dgo_fixture_wide.argtypes = [VP, VP]
+    lib.dgo_fixture_model_attn.argtypes = [C.c_uint32] * 5 + [VP, VP]
+    lib.dgo_fixture_model_full.argtypes = [C.c_uint32] * 5 + [VP, VP]
+    lib.dgo_synthetic_fill_kv.argtypes = [VP, C.c_size_t, C.c_uint64]
+    lib.dgo_max_threads.restype = C.c_int
+    _lib = lib
+    return lib
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def make_desc(canvas, n_q_heads, n_kv_heads, head_dim, kv_len, *, causal_rows=0, window=0, kv_ring_mask=0,
+              causal_sees_masked=0, strict_order=0, t_lo_override=-1, scale=1.0, layout="reference", t_cap=None):
+    d = Desc(canvas=canvas, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, head_dim=head_dim, kv_len=kv_len,
+             causal_rows=causal_rows, window=window, kv_ring_mask=kv_ring_mask,
+             causal_sees_masked=causal_sees_masked, strict_order=strict_order, t_lo_override=t_lo_override,
+             scale=scale)
+    lib = load()
+    if layout == "reference":
+        lib.dgo_desc_reference_layout(C.byref(d))
+    elif layout == "head_major":
+        lib.dgo_desc_head_major_layout(C.byref(d), t_cap if t_cap is not None else kv_len + canvas)
+    else:
+        raise ValueError(layout)
+    return d
+
+
+def _toks(tok_list):
+    if tok_list is None:
+        return None, 0
+    t = np.ascontiguousarray(tok_list, dtype=np.uint32)
+    return t, len(t)
+
+
+def attention_f32(desc, q, kv, tok_list=None, n_threads=0):
+    """Returns (out [canvas,Hq,hd] f32, lse [canvas,Hq] f32); rows not in tok_list stay 0."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    kv = np.ascontiguousarray(kv, dtype=np.float32)
+    out = np.zeros((desc.canvas, desc.n_q_heads, desc.head_dim), dtype=np.float32)
+    lse = np.zeros((desc.canvas, desc.n_q_heads), dtype=np.float32)
+    t, n = _toks(tok_list)
+    load().dgo_attention_f32(C.byref(desc), _ptr(q), _ptr(kv), _ptr(out), _ptr(lse), _ptr(t), n, n_threads)
+    return out, lse
+
+
+def attention_f64(desc, q, kv, tok_list=None, n_threads=0):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    kv = np.ascontiguousarray(kv, dtype=np.float32)
+    out = np.zeros((desc.canvas, desc.n_q_heads, desc.head_dim), dtype=np.float64)
+    lse = np.zeros((desc.canvas, desc.n_q_heads), dtype=np.float64)
+    t, n = _toks(tok_list)
+    load().dgo_attention_f64(C.byref(desc), _ptr(q), _ptr(kv), _ptr(out), _ptr(lse), _ptr(t), n, n_threads)
+    return out, lse
+
+
+def attention_blocked_f32(desc, q, kv, bk, n_threads=0):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    kv = np.ascontiguousarray(kv, dtype=np.float32)
+    out = np.zeros((desc.canvas, desc.n_q_heads, desc.head_dim), dtype=np.float32)
+    lse = np.zeros((desc.canvas, desc.n_q_heads), dtype=np.float32)
+    load().dgo_attention_blocked_f32(C.byref(desc), _ptr(q), _ptr(kv), _ptr(out), _ptr(lse), bk, n_threads)
+    return out, lse
+
+
+def attention_partial_f32(desc, q, kv, t_begin, t_end, n_threads=0):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    kv = np.ascontiguousarray(kv, dtype=np.float32)
+    rows = desc.canvas * desc.n_q_heads
+    acc = np.zeros((rows, desc.head_dim), dtype=np.float32)
+    m = np.zeros(rows, dtype=np.float32)
+    l = np.zeros(rows, dtype=np.float32)
+    load().dgo_attention_partial_f32(C.byref(desc), _ptr(q), _ptr(kv), t_begin, t_end, _ptr(acc), _ptr(m), _ptr(l),
+                                     n_threads)
+    return acc, m, l
+
+
+def merge_partials_f32(parts, head_dim):
+    """parts: list of (acc [rows,hd], m [rows], l [rows])."""
+    n = len(parts)
+    rows = parts[0][1].shape[0]
+    arr = lambda i: (C.c_void_p * n)(*[p[i].ctypes.data for p in parts])
+    out = np.zeros((rows, head_dim), dtype=np.float32)
+    lse = np.zeros(rows, dtype=np.float32)
+    load().dgo_merge_partials_f32(rows, head_dim, n, arr(0), arr(1), arr(2), _ptr(out), _ptr(lse))
+    return out, lse
+
+
+def attention_bitmap_f32(q, k, v, mask, n_heads, n_kv_heads, head_dim):
+    """q [seq,Hq,hd], k/v [total_kv,Hkv,hd], mask [seq,total_kv] bool."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    mask = np.ascontiguousarray(mask, dtype=np.uint8)
+    seq, total = mask.shape
+    out = np.zeros((seq, n_heads, head_dim), dtype=np.float32)
+    load().dgo_attention_bitmap_f32(seq, total, n_heads, n_kv_heads, head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask),
+                                    _ptr(out))
+    return out
+
+
+def visible_matrix(desc):
+    lib = load()
+    t_all = desc.kv_len + desc.canvas
+    m = np.zeros((desc.canvas, t_all), dtype=bool)
+    for tok in range(desc.canvas):
+        for t in range(t_all):
+            m[tok, t] = bool(lib.dgo_visible(C.byref(desc), tok, t))
+    return m
+
+
+ROUND_BF16_TRUNC, ROUND_BF16_RNE, ROUND_F16_TRUNC, ROUND_F16_RNE = 0, 1, 2, 3
+
+
+def round_array(x, mode):
+    y = np.array(x, dtype=np.float32, copy=True, order="C")
+    load().dgo_round_array(_ptr(y), y.size, mode)
+    return y
+
+
+def to_bits(x, mode):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    b = np.zeros(x.shape, dtype=np.uint16)
+    load().dgo_to_bits(_ptr(x), _ptr(b), x.size, mode)
+    return b
+
+
+def from_bits(b, is_f16):
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    x = np.zeros(b.shape, dtype=np.float32)
+    load().dgo_from_bits(_ptr(b), _ptr(x), b.size, 1 if is_f16 else 0)
+    return x
+
+
+def rms_norm_no_scale(x, eps=1e-6):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros_like(x)
+    load().dgo_rms_norm_no_scale(_ptr(out), _ptr(x), x.size, eps)
+    return out
+
+
+def fixture(name, *dims):
+    """Reference fixture generators; returns (q, kv) flat f32 arrays."""
+    lib = load()
+    if name == "tiny":
+        q, kv = np.zeros(2 * 4 * 32, np.float32), np.zeros(4 * 2 * 32 * 2, np.float32)
+        lib.dgo_fixture_tiny(_ptr(q), _ptr(kv))
+    elif name == "wide":
+        q, kv = np.zeros(4 * 8 * 64, np.float32), np.zeros(8 * 2 * 64 * 2, np.float32)
+        lib.dgo_fixture_wide(_ptr(q), _ptr(kv))
+    elif name in ("model_attn", "model_full"):
+        canvas, nq, nkv, hd, kv_len = dims
+        q = np.zeros(canvas * nq * hd, np.float32)
+        kv = np.zeros((kv_len + canvas) * nkv * hd * 2, np.float32)
+        getattr(lib, "dgo_fixture_" + name)(canvas, nq, nkv, hd, kv_len, _ptr(q), _ptr(kv))
+    else:
+        raise ValueError(name)
+    return q, kv
+
+
+def synthetic_fill_kv(n, seed):
+    b = np.zeros(n, dtype=np.uint16)
+    load().dgo_synthetic_fill_kv(_ptr(b), n, seed)
+    return b
+
+
+def max_threads():
+    return load().dgo_max_threads()
