@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the denoise-step attention on one MI355X.
+
+One step = one dg_attn_forward call (main MFMA kernel + split merge) over one synthetic
+batch already resident in HBM.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3_global] [--no-cpu-baseline]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg3_global")
+    ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline sample time")
+    ap.add_argument("--check-toks", type=int, default=12)
+    return ap.parse_args()
+
+
+def cpu_baseline(w, q, kv, flops_per_tok, seconds):
+    """Times the oracle (a port of the reference's CPU attention) on a bounded sample of canvas rows."""
+    from oracle import pyoracle as po
+    d = po.make_desc(w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, causal_rows=w.causal_rows,
+                     window=w.window, causal_sees_masked=1 if w.sees_masked else 0,
+                     t_lo_override=-1 if w.t_lo is None else w.t_lo, layout=w.layout, t_cap=w.t_all)
+    threads = min(po.max_threads(), 16)
+    # calibrate on a few bidirectional rows (the most expensive kind), then size the sample
+    probe = np.arange(w.canvas - 2, w.canvas, dtype=np.uint32)
+    t0 = time.perf_counter()
+    po.attention_f32(d, q, kv, tok_list=probe, n_threads=threads)
+    dt = max(time.perf_counter() - t0, 1e-4)
+    n = int(max(2, min(w.canvas, round(seconds / (dt / len(probe))))))
+    toks = np.unique(np.linspace(0, w.canvas - 1, n).round().astype(np.uint32))
+    t0 = time.perf_counter()
+    po.attention_f32(d, q, kv, tok_list=toks, n_threads=threads)
+    dt = time.perf_counter() - t0
+    fl = float(sum(flops_per_tok[t] for t in toks))
+    return {"value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{len(toks)} of {w.canvas} canvas rows (evenly spaced) x all {w.n_q_heads} heads, "
+                      f"{dt:.2f} s, fp32 online-softmax port of the reference CPU attention, OpenMP"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible; the attention path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    from diffgemma_amd import attention as A, capi, workloads as W
+    from oracle import pyoracle as po
+
+    w = W.config(args.workload)
+    t_gen = time.perf_counter()
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+    t_gen = time.perf_counter() - t_gen
+    desc = w.desc(n_splits=args.splits)
+    pairs, flops = capi.visible_pairs(desc)
+    n_splits = capi.resolved_splits(desc)
+    out_dt = torch.int16 if w.dtype == "bf16" else torch.float32
+    out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=out_dt, device="cuda")
+    lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+    ws = A.alloc_workspace(desc)
+
+    # ---- correctness against the oracle on a row sample, before anything is timed ----
+    A.forward(desc, qd, kd, out, lse, ws)
+    torch.cuda.synchronize()
+    od = po.make_desc(w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, causal_rows=w.causal_rows,
+                      window=w.window, causal_sees_masked=1 if w.sees_masked else 0,
+                      t_lo_override=-1 if w.t_lo is None else w.t_lo, layout=w.layout, t_cap=w.t_all)
+    toks = np.unique(np.concatenate([
+        np.linspace(0, w.canvas - 1, max(2, args.check_toks)).round().astype(np.uint32),
+        np.array([max(w.causal_rows, 1) - 1, min(w.causal_rows, w.canvas - 1)], dtype=np.uint32)]))
+    ref, ref_lse = po.attention_f32(od, q, kv, tok_list=toks)
+    if w.dtype == "bf16":
+        from diffgemma_amd import rounding as R
+        got = R.bf16_bits_to_f32(out.cpu().numpy().view(np.uint16)).reshape(w.canvas, w.n_q_heads, w.head_dim)
+    else:
+        got = out.cpu().numpy().reshape(w.canvas, w.n_q_heads, w.head_dim)
+    got_lse = lse.cpu().numpy().reshape(w.canvas, w.n_q_heads)
+    diff = np.abs(got[toks] - ref[toks])
+    lse_rel = np.abs(got_lse[toks] - ref_lse[toks]) / np.maximum(np.abs(ref_lse[toks]), 1e-6)
+    check = {"rows": int(len(toks)), "max_abs": float(diff.max()), "mean_abs": float(diff.mean()),
+             "lse_rel_max": float(lse_rel.max()), "tol": {"max_abs": 2e-2, "mean_abs": 2e-3, "lse_rel": 1e-3}}
+    check["passed"] = bool(diff.max() <= 2e-2 and diff.mean() <= 2e-3 and lse_rel.max() <= 1e-3
+                           and np.isfinite(got).all())
+
+    # ---- warm-up, then exactly K timed steps ----
+    for _ in range(args.warmup):
+        A.forward(desc, qd, kd, out, lse, ws)
+    torch.cuda.synchronize()
+    capi.prof_begin(args.steps)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        A.forward(desc, qd, kd, out, lse, ws)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kern_ms_total, n_rec = capi.prof_end()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    kern_ms = kern_ms_total / max(n_rec, 1)
+
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    kern_tflops = flops / (kern_ms * 1e-3) / 1e12
+    kv_bytes = 2 * w.n_kv_heads * w.head_dim * 2 * (pairs // w.canvas if w.window else w.t_all)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.workload)
+        except Exception:
+            traffic = None
+
+    res = {
+        "metric": "denoise attention TFLOP/s + % bf16 MFMA peak, 256-canvas @ 32k prefix, 1 GPU",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == "bf16" else "f16", "data": "synthetic",
+        "config": {"workload": w.name, "canvas": w.canvas, "kv_prefix": w.kv_len, "n_q_heads": w.n_q_heads,
+                   "n_kv_heads": w.n_kv_heads, "head_dim": w.head_dim, "causal_rows": w.causal_rows,
+                   "window": w.window, "kv_layout": w.layout, "n_splits": n_splits,
+                   "mask": "rows<causal_rows causal in canvas, rest bidirectional; prefix all-visible"
+                           if not w.window else "sliding window, reference rule t_lo=kv_len-(window-1)"},
+        "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
+        "canvas_tokens_per_s": w.canvas / (ms_per_step * 1e-3),
+        "flops_per_step": flops, "visible_pairs_per_head": pairs,
+        "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": kern_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
+                     "kernel": "attn_mfma_kernel", "kernel_ms": kern_ms,
+                     "kv_gbs": kv_bytes / (kern_ms * 1e-3) / 1e9, "hbm_peak_gbs": PEAK_HBM_GBS},
+        "check": check, "input_gen_s": t_gen,
+    }
+    if not args.no_cpu_baseline:
+        # per-row FLOPs (rows differ under the causal part of the mask)
+        t_all = w.t_all
+        per_row_pairs = np.zeros(w.canvas, dtype=np.int64)
+        for t in range(w.canvas):
+            causal = t < w.causal_rows
+            qpos = w.kv_len + t
+            hi = min(t_all, qpos + 1) if causal else t_all
+            if w.window:
+                anchor = qpos if causal else w.kv_len
+                lo = max(0, anchor - (w.window - 1))
+            else:
+                lo = 0
+            if not causal and w.t_lo is not None:
+                lo = w.t_lo
+            n = max(0, hi - lo)
+            if causal and w.sees_masked:
+                n += max(0, t_all - max(w.kv_len + w.causal_rows, hi))
+            per_row_pairs[t] = n
+        assert int(per_row_pairs.sum()) == pairs, (int(per_row_pairs.sum()), pairs)
+        per_tok = {t: 4.0 * w.head_dim * w.n_q_heads * float(per_row_pairs[t]) for t in range(w.canvas)}
+        res["cpu_baseline"] = cpu_baseline(w, q, kv, per_tok, args.cpu_seconds)
+    print(json.dumps(res), flush=True)
+    if not check["passed"]:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

@@ -23,7 +23,7 @@ EXPORTS = (
     "dg_attn_desc_reference_layout", "dg_attn_desc_head_major_layout", "dg_attn_workspace_bytes",
     "dg_attn_resolved_splits", "dg_attn_forward", "dg_attn_strerror", "dg_attn_abi_version",
     "dg_attn_visible_pairs", "dg_attention_dispatch", "dg_attention_state_bytes", "dg_kv_row_bytes",
-    "dg_kv_region_bytes", "dg_kv_slot", "dg_layer_kv_slots",
+    "dg_kv_region_bytes", "dg_kv_slot", "dg_layer_kv_slots", "dg_prof_begin", "dg_prof_end",
 )
 
 
@@ -122,6 +122,10 @@ def load():
     lib.dg_kv_slot.restype = C.c_uint64
     lib.dg_layer_kv_slots.argtypes = [C.c_int, C.c_uint64, C.c_uint64]
     lib.dg_layer_kv_slots.restype = C.c_uint64
+    lib.dg_prof_begin.argtypes = [C.c_uint32]
+    lib.dg_prof_begin.restype = C.c_int
+    lib.dg_prof_end.argtypes = [P(C.c_double), P(C.c_uint32)]
+    lib.dg_prof_end.restype = C.c_int
     _lib = lib
     return lib
 
@@ -151,3 +155,14 @@ def visible_pairs(desc: AttnDesc):
     n, f = C.c_uint64(0), C.c_double(0.0)
     check(load().dg_attn_visible_pairs(C.byref(desc), C.byref(n), C.byref(f)))
     return n.value, f.value
+
+
+def prof_begin(max_launches: int) -> None:
+    check(load().dg_prof_begin(max_launches))
+
+
+def prof_end():
+    """Returns (summed main-kernel ms, launches recorded)."""
+    ms, n = C.c_double(0.0), C.c_uint32(0)
+    check(load().dg_prof_end(C.byref(ms), C.byref(n)))
+    return ms.value, n.value

@@ -122,7 +122,9 @@ __device__ __forceinline__ void issue_tile(const char* head_base, int64_t tok_st
   }
 }
 
-template <int D, bool F16>
+// PIPE: issue Q.K^T of tile j+1 before the softmax of tile j (needs a second score tile in
+// registers; used where the register file has room for it).
+template <int D, bool F16, bool PIPE>
 __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   constexpr int CPR = D / 8, ROWB = 2 * D, TILEB = kBlockN * ROWB, NSTEP = D / 16, NDB = D / 32;
   __shared__ __attribute__((aligned(1024))) char sk0[TILEB];
@@ -248,23 +250,35 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     issue_tile<D, true>(vbase, vstride_b, tb * kBlockN, p.t_all, p.ring_mask, v0, wave, lane);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    f32x16 s_cur = qk_tile(k0);
+    f32x16 s_cur;
+    if constexpr (PIPE) s_cur = qk_tile(k0);
 
     for (uint32_t jj = 0; jj < ntile; ++jj) {
       const uint32_t t0 = (tb + jj) * kBlockN;
-      lds_char* const kb_next = (jj & 1u) ? k0 : k1;   // holds K(jj+1)
-      lds_char* const kb_free = (jj & 1u) ? k1 : k0;   // held K(jj): refill with K(jj+2)
+      lds_char* const kb_even = (jj & 1u) ? k1 : k0;   // holds K(jj)
+      lds_char* const kb_odd = (jj & 1u) ? k0 : k1;    // holds K(jj+1)
       lds_char* const vb_cur = (jj & 1u) ? v1 : v0;    // holds V(jj)
       lds_char* const vb_free = (jj & 1u) ? v0 : v1;   // refill with V(jj+1)
 
-      // K(jj+1) and V(jj) have landed everywhere; every wave is done with the previous tile.
+      // The tiles this iteration reads have landed everywhere, and every wave is done with
+      // the buffers about to be refilled.
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (jj + 2 < ntile) issue_tile<D, false>(kbase, kstride_b, t0 + 2 * kBlockN, p.t_all, p.ring_mask, kb_free, wave, lane);
+      if constexpr (PIPE) {
+        // K(jj) was consumed one iteration ago: its buffer takes K(jj+2)
+        if (jj + 2 < ntile) issue_tile<D, false>(kbase, kstride_b, t0 + 2 * kBlockN, p.t_all, p.ring_mask, kb_even, wave, lane);
+      } else {
+        // K(jj+1) goes to the other buffer (prologue loaded K(tb+1) already for jj == 0)
+        if (jj >= 1 && jj + 1 < ntile) issue_tile<D, false>(kbase, kstride_b, t0 + kBlockN, p.t_all, p.ring_mask, kb_odd, wave, lane);
+      }
       if (jj + 1 < ntile) issue_tile<D, true>(vbase, vstride_b, t0 + kBlockN, p.t_all, p.ring_mask, vb_free, wave, lane);
 
       f32x16 s_next;
-      if (jj + 1 < ntile) s_next = qk_tile(kb_next);
+      if constexpr (PIPE) {
+        if (jj + 1 < ntile) s_next = qk_tile(kb_odd);
+      } else {
+        s_cur = qk_tile(kb_even);
+      }
 
       // ---- mask (edge tiles only) ----
       const bool masked = !(t0 >= lo_max && t0 + kBlockN <= hi_min);
@@ -284,8 +298,21 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         const float m_new = fmaxf(m_ref, tmax);
         const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
         l_part *= corr;
+        // O lives in accumulator registers, which only MFMA and the accvgpr moves can touch.
+        // Spelling the multiply out keeps the values in that register class on both sides
+        // of this rarely taken branch; a plain `o[i] *= corr` makes the allocator shuttle
+        // all of O through VGPRs and spill.
 #pragma unroll
-        for (int i = 0; i < NDB; ++i) o[i] *= corr;
+        for (int i = 0; i < NDB; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            float tmp;
+            float x = o[i][e];
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                         : "+a"(x), "=&v"(tmp)
+                         : "v"(corr));
+            o[i][e] = x;
+          }
         m_ref = m_new;
       }
       const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
@@ -318,7 +345,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           o[db] = mfma16<F16>(a, pf[ks], o[db]);
         }
       }
-      if (jj + 1 < ntile) s_cur = s_next;
+      if constexpr (PIPE) {
+        if (jj + 1 < ntile) s_cur = s_next;
+      }
     }
   }
 
@@ -375,7 +404,8 @@ template <int D, bool F16>
 hipError_t launch_one(const AttnParams& p, hipStream_t s) {
   const uint32_t nstream = p.hkv * p.n_splits;
   const uint32_t grid = ((nstream + 7u) / 8u) * p.n_mtiles * 8u;
-  hipLaunchKernelGGL((attn_mfma_kernel<D, F16>), dim3(grid), dim3(256), 0, s, p);
+  constexpr bool kPipe = D < 512;  // at D=512 the second score tile does not fit next to O and Q
+  hipLaunchKernelGGL((attn_mfma_kernel<D, F16, kPipe>), dim3(grid), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 

@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "attn_params.h"
 
@@ -26,6 +27,13 @@ struct DeviceInfo {
 DeviceInfo g_dev[64];
 thread_local uint32_t* g_tls_dbg = nullptr;
 std::mutex g_dev_mu;
+
+struct ProfState {
+  std::vector<hipEvent_t> ev;
+  uint32_t used = 0;
+  bool active = false;
+};
+thread_local ProfState g_prof;
 
 int device_info(DeviceInfo* out) {
   int dev = 0;
@@ -330,7 +338,13 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
     if (dg::launch_attn_scalar(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
     return DG_OK;
   }
+  const bool prof = g_prof.active && 2 * (size_t)g_prof.used + 1 < g_prof.ev.size();
+  if (prof) (void)hipEventRecord(g_prof.ev[2 * g_prof.used], s);
   if (dg::launch_attn_mfma(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+  if (prof) {
+    (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 1], s);
+    ++g_prof.used;
+  }
   if (pl.n_splits > 1 && dg::launch_attn_merge(p, hd, s) != hipSuccess) return DG_ERR_LAUNCH;
   return DG_OK;
 }
@@ -371,6 +385,36 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
   g_tls_dbg = (uint32_t*)dbg;
   const int rc = dg_attn_forward(&d, q, kvcache, out, nullptr, attn_state, attn_state_bytes, stream);
   g_tls_dbg = nullptr;
+  return rc;
+}
+
+int dg_prof_begin(uint32_t max_launches) {
+  if (g_prof.active) return DG_ERR_UNSUPPORTED;
+  g_prof.ev.assign(2 * (size_t)max_launches, nullptr);
+  for (auto& e : g_prof.ev)
+    if (hipEventCreate(&e) != hipSuccess) return DG_ERR_LAUNCH;
+  g_prof.used = 0;
+  g_prof.active = true;
+  return DG_OK;
+}
+
+int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches) {
+  if (!g_prof.active) return DG_ERR_UNSUPPORTED;
+  double total = 0.0;
+  int rc = DG_OK;
+  if (g_prof.used > 0 && hipEventSynchronize(g_prof.ev[2 * g_prof.used - 1]) != hipSuccess) rc = DG_ERR_LAUNCH;
+  for (uint32_t i = 0; i < g_prof.used && rc == DG_OK; ++i) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]) != hipSuccess) rc = DG_ERR_LAUNCH;
+    total += ms;
+  }
+  for (auto e : g_prof.ev)
+    if (e) (void)hipEventDestroy(e);
+  if (main_kernel_ms_total) *main_kernel_ms_total = total;
+  if (n_launches) *n_launches = g_prof.used;
+  g_prof.ev.clear();
+  g_prof.used = 0;
+  g_prof.active = false;
   return rc;
 }
 

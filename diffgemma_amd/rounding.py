@@ -16,10 +16,12 @@ def f32_to_bf16_bits_trunc(x: np.ndarray) -> np.ndarray:
 
 
 def f32_to_bf16_bits_rne(x: np.ndarray) -> np.ndarray:
-    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
-    nan = (u & 0x7FFFFFFF) > 0x7F800000
-    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
-    r = np.where(nan, (u >> 16) | 0x40, r)
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    with np.errstate(over="ignore"):  # only NaN patterns can wrap, and those are replaced below
+        r = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    if nan.any():
+        r = np.where(nan, (u >> np.uint32(16)) | np.uint32(0x40), r)
     return r.astype(np.uint16)
 
 

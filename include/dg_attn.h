@@ -159,6 +159,15 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
 int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
                              size_t* out_bytes);
 
+/* ---- optional kernel timing (measurement aid; no counterpart in the reference, whose
+ * harness times whole command buffers: src/shaders/attn/harness.rs:149-170) ----
+ * Between dg_prof_begin and dg_prof_end every dg_attn_forward issued by the calling thread
+ * records one HIP event pair on its stream around the main attention kernel only (the
+ * merge and conversion kernels stay outside the pair).  dg_prof_end waits for the last
+ * recorded event, returns the summed kernel time and releases the events. */
+int dg_prof_begin(uint32_t max_launches);
+int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches);
+
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);
 uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slots, uint32_t kv_dtype);
