@@ -1,0 +1,385 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on identical
+seeded inputs.  Tolerances: the reference's per-fixture ones (attention/mod.rs:846-946:
+max_abs 1e-2 / 2e-2, cosine >= 0.9999) on its own fixtures; max-abs <= 2e-2, mean-abs <= 2e-3
+on bf16 outputs and per-row LSE within 1e-3 relative on the benchmark configurations."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from diffgemma_amd import attention as A
+from diffgemma_amd import capi, rounding as R, workloads as W
+from helpers import assert_oracle, max_abs_diff, mean_abs_diff
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS, LSE_REL = 2e-2, 2e-3, 1e-3
+
+FIXTURES = {
+    "tiny": (A.tiny_fixture, 1e-2), "wide": (A.wide_fixture, 2e-2), "full_hd512": (A.full_hd512_fixture, 2e-2),
+    "full_grp8_hd512": (A.full_grp8_hd512_fixture, 2e-2), "sliding_hd256": (A.sliding_hd256_fixture, 2e-2),
+}
+
+
+def reference_cpu(po, f, **kw):
+    """The reference's test wrapper (attention/mod.rs:218-240): Q -> bf16, KV -> f16, both by
+    truncation; run the oracle; output -> bf16 by truncation."""
+    q = R.bf16_bits_to_f32(R.f32_to_bf16_bits_trunc(f.q))
+    kv = R.f16_bits_to_f32(R.f32_to_f16_bits_trunc(f.kvcache))
+    d = po.make_desc(f.canvas, f.n_q_heads, f.n_kv(), f.head_dim(), f.kv_len, **kw)
+    out, lse = po.attention_f32(d, q, kv)
+    return po.round_array(out, po.ROUND_BF16_TRUNC).ravel(), out.ravel(), lse.ravel()
+
+
+# ------------------------------------------------------------------ the reference's Tier-1 matrix
+@pytest.mark.parametrize("name", list(FIXTURES))
+def test_reference_fixture_scalar_kernel(gpu_ready, po, name):
+    fn, tol = FIXTURES[name]
+    f = fn()
+    want, _, _ = reference_cpu(po, f)
+    assert_oracle(A.gpu(f), want, tol, 0.9999)
+
+
+@pytest.mark.parametrize("name", list(FIXTURES))
+@pytest.mark.parametrize("causal", [0, 1])
+def test_reference_fixture_mfma_dispatch(gpu_ready, po, name, causal):
+    """Through dg_attention_dispatch: the buffers encode_layer_attention_dispatch binds."""
+    fn, tol = FIXTURES[name]
+    f = fn()
+    want, _, _ = reference_cpu(po, f, causal_rows=f.canvas if causal else 0)
+    rig = A.AttnRig.from_fixture(f)
+    rig.run_dispatch(causal=causal)
+    assert_oracle(rig.read_out_f32(), want, tol, 0.9999)
+    assert rig.read_debug_status().code == 0
+
+
+@pytest.mark.parametrize("name", list(FIXTURES))
+def test_reference_fixture_unrounded_and_lse(gpu_ready, po, name):
+    import torch
+    f = FIXTURES[name][0]()
+    _, want, want_lse = reference_cpu(po, f)
+    rig = A.AttnRig.from_fixture(f)
+    d = rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=False)
+    d.out_dtype = capi.DG_F32
+    out = torch.zeros(f.out_len(), dtype=torch.float32, device="cuda")
+    A.forward(d, rig.buf_q, rig.buf_kv, out, rig.buf_lse, rig.workspace_for(d))
+    torch.cuda.synchronize()
+    assert max_abs_diff(out.cpu().numpy(), want) < 2e-4
+    lse = rig.read_lse()
+    assert np.max(np.abs(lse - want_lse) / np.maximum(np.abs(want_lse), 1.0)) < LSE_REL
+
+
+def test_model_full_fixture_midsize(gpu_ready, po):
+    """The reference's bench fixture (attention_gemm/mod.rs:364-432) at a prefix that spans many key tiles."""
+    f = A.model_full_fixture(1000, canvas=64)
+    want, _, _ = reference_cpu(po, f)
+    assert_oracle(A.gpu_mma(f), want, 2e-2, 0.9999)
+
+
+# ------------------------------------------------------------------ generic runner
+def run_workload(po, w, *, n_splits=0, kernel=capi.DG_KERNEL_AUTO, out_f32=False, toks=None, ring=None, flags=0,
+                 kv_override=None):
+    import torch
+    q, kv = W.generate(w)
+    if kv_override is not None:
+        kv = kv_override(kv)
+    qd, kd = W.device_arrays(w, q, kv)
+    desc = w.desc(n_splits=n_splits, kernel=kernel, flags=flags)
+    if out_f32:
+        desc.out_dtype = capi.DG_F32
+    is_bf16_out = desc.out_dtype == capi.DG_BF16
+    out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.int16 if is_bf16_out else torch.float32,
+                      device="cuda")
+    lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+    A.forward(desc, qd, kd, out, lse, A.alloc_workspace(desc))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    got = R.bf16_bits_to_f32(got.view(np.uint16)) if is_bf16_out else got
+    got = got.reshape(w.canvas, w.n_q_heads, w.head_dim)
+    got_lse = lse.cpu().numpy().reshape(w.canvas, w.n_q_heads)
+    od = po.make_desc(w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, causal_rows=w.causal_rows,
+                      window=w.window, causal_sees_masked=1 if w.sees_masked else 0,
+                      t_lo_override=-1 if w.t_lo is None else w.t_lo, layout=w.layout, t_cap=w.t_all)
+    ref, ref_lse = po.attention_f32(od, q, kv, tok_list=toks)
+    rows = np.arange(w.canvas) if toks is None else np.asarray(toks)
+    return got[rows], got_lse[rows], ref[rows], ref_lse[rows]
+
+
+def check_tolerances(got, got_lse, ref, ref_lse, max_abs=MAX_ABS, mean_abs=MEAN_ABS):
+    assert np.all(np.isfinite(got))
+    assert max_abs_diff(got, ref) <= max_abs
+    assert mean_abs_diff(got, ref) <= mean_abs
+    assert np.max(np.abs(got_lse - ref_lse) / np.maximum(np.abs(ref_lse), 1e-6)) <= LSE_REL
+
+
+# ------------------------------------------------------------------ benchmark configurations
+def test_cfg1_tiny_fp32(gpu_ready, po):
+    """fp32 in, fp32 out; the library computes in f16 after a conversion pass."""
+    got, lse, ref, ref_lse = run_workload(po, W.config("cfg1_tiny"))
+    check_tolerances(got, lse, ref, ref_lse, max_abs=2e-4, mean_abs=2e-5)
+
+
+@pytest.mark.parametrize("name", ["cfg2_sliding", "cfg2_sliding_768"])
+def test_cfg2_sliding_window(gpu_ready, po, name):
+    check_tolerances(*run_workload(po, W.config(name)))
+
+
+@pytest.mark.parametrize("name", ["cfg3_global", "cfg3_global_b"])
+def test_cfg3_global_full_size(gpu_ready, po, name):
+    """Full 32k-prefix shape, every row, mixed committed/bidirectional mask."""
+    check_tolerances(*run_workload(po, W.config(name)))
+
+
+def test_cfg3_unrounded_output_error_budget(gpu_ready, po):
+    """fp32 output isolates the kernel's own error (bf16 probabilities) from output rounding."""
+    toks = np.arange(0, 256, 5, dtype=np.uint32)
+    got, lse, ref, ref_lse = run_workload(po, W.config("cfg3_global"), out_f32=True, toks=toks)
+    check_tolerances(got, lse, ref, ref_lse, max_abs=8e-3, mean_abs=3e-4)
+
+
+def test_cfg4_long_context_rows(gpu_ready, po):
+    """131072-key prefix with 1% of keys scaled x8 (peaked rows); oracle on a row sample."""
+    toks = np.array([0, 1, 63, 64, 127, 128, 200, 255], dtype=np.uint32)
+    check_tolerances(*run_workload(po, W.config("cfg4_long"), toks=toks))
+
+
+def test_cfg5_sliding_layer_at_32k(gpu_ready, po):
+    check_tolerances(*run_workload(po, W.config("cfg5_sliding_32k")))
+
+
+# ------------------------------------------------------------------ size-independent properties at full size
+def _device_run(w, q, kv, **kw):
+    import torch
+    qd, kd = W.device_arrays(w, q, kv)
+    desc = w.desc(**kw)
+    desc.out_dtype = capi.DG_F32
+    out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.float32, device="cuda")
+    lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+    A.forward(desc, qd, kd, out, lse, A.alloc_workspace(desc))
+    torch.cuda.synchronize()
+    return out.cpu().numpy().reshape(w.canvas, w.n_q_heads, w.head_dim), lse.cpu().numpy().reshape(w.canvas, -1)
+
+
+def test_split_count_invariance_full_size(gpu_ready):
+    """Split-KV + LSE merge: any split count gives the single-pass result (cfg 3 shape)."""
+    w = W.config("cfg3_global")
+    q, kv = W.generate(w)
+    base, base_lse = _device_run(w, q, kv, n_splits=1)
+    for s in (2, 8, 13, 64):
+        out, lse = _device_run(w, q, kv, n_splits=s)
+        assert max_abs_diff(out, base) < 1.6e-2 and mean_abs_diff(out, base) < 4e-4, s   # two bf16-P roundings
+        assert np.max(np.abs(lse - base_lse) / np.abs(base_lse)) < 1e-4, s
+
+
+def test_scalar_and_mfma_kernels_agree_full_size(gpu_ready):
+    w = W.scaled(W.config("cfg3_global"), 8192)
+    q, kv = W.generate(w)
+    a, la = _device_run(w, q, kv, kernel=capi.DG_KERNEL_SCALAR)
+    b, lb = _device_run(w, q, kv, kernel=capi.DG_KERNEL_MFMA)
+    assert max_abs_diff(a, b) < 8e-3 and mean_abs_diff(a, b) < 3e-4
+    assert np.max(np.abs(la - lb) / np.abs(la)) < 1e-4
+
+
+def test_constant_value_rows_pass_through(gpu_ready):
+    """If every key's V row is the same vector the output is that vector, whatever the scores."""
+    w = W.config("cfg3_global")
+    q, kv = W.generate(w)
+    vrow = kv[1, :, :1, :].copy()
+    kv[1] = vrow
+    out, _ = _device_run(w, q, kv)
+    want = np.repeat(vrow[:, 0, :], w.n_q_heads // w.n_kv_heads, axis=0)[None]
+    assert max_abs_diff(out, np.broadcast_to(want, out.shape)) < 1e-5 + 4e-3 * np.abs(vrow).max()
+
+
+def test_linearity_in_v_full_size(gpu_ready):
+    """out(V1 + V2) = out(V1) + out(V2) for fixed Q, K."""
+    w = W.scaled(W.config("cfg3_global"), 16384)
+    q, kv = W.generate(w)
+    rng = np.random.default_rng(99)
+    v2 = R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(rng.standard_normal(kv[1].shape).astype(np.float32) * 0.5)).reshape(kv[1].shape)
+    kv1, kv2, kv12 = kv.copy(), kv.copy(), kv.copy()
+    kv2[1] = v2
+    kv12[1] = R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(kv[1] + v2)).reshape(v2.shape)
+    o1, _ = _device_run(w, q, kv1)
+    o2, _ = _device_run(w, q, kv2)
+    o12, _ = _device_run(w, q, kv12)
+    # bf16 rounding of V1+V2 costs up to 2^-9 relative per element
+    assert max_abs_diff(o12, o1 + o2) < 3e-2 and mean_abs_diff(o12, o1 + o2) < 3e-3
+
+
+def test_gqa_group_shares_keys(gpu_ready):
+    """Heads of one group fed the same Q row produce the same output (kvh = qh / group)."""
+    w = W.scaled(W.config("cfg3_global"), 2048)
+    q, kv = W.generate(w)
+    q[:] = q[:, :1, :]
+    out, lse = _device_run(w, q, kv)
+    for h in range(1, 8):
+        assert np.array_equal(out[:, h], out[:, 0]) and np.array_equal(lse[:, h], lse[:, 0])
+    assert max_abs_diff(out[:, 8], out[:, 0]) > 1e-3
+
+
+# ------------------------------------------------------------------ edge cases
+CASES = [
+    # canvas, hq, hkv, hd, kv_len, causal_rows, window, splits
+    (1, 4, 2, 64, 0, 0, 0, 0),          # single row, no prefix
+    (1, 16, 2, 512, 77, 1, 0, 0),       # single causal row
+    (64, 16, 8, 256, 100, 0, 0, 0),     # retry canvas 64
+    (128, 16, 2, 512, 500, 64, 0, 0),   # retry canvas 128, mixed mask
+    (256, 16, 8, 256, 0, 256, 0, 0),    # prefill from an empty cache
+    (37, 16, 8, 256, 333, 20, 100, 2),  # ragged everything
+    (256, 8, 4, 128, 512, 0, 0, 0),     # hd 128
+    (256, 16, 8, 256, 5000, 256, 1024, 0),  # causal sliding prefill
+    (33, 6, 3, 32, 95, 0, 40, 3),       # hd 32, group 2
+    (200, 12, 4, 64, 1, 100, 0, 0),     # group 3, one prefix key
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_edge_cases(gpu_ready, po, case):
+    c, hq, hkv, hd, kvl, cr, win, splits = case
+    w = W.Workload("edge", c, hq, hkv, hd, kvl, causal_rows=cr, window=win, seed=hash(case) & 0xFFFF)
+    check_tolerances(*run_workload(po, w, n_splits=splits))
+    check_tolerances(*run_workload(po, w, kernel=capi.DG_KERNEL_SCALAR))
+
+
+def test_reference_layout_equals_head_major(gpu_ready):
+    w = W.Workload("lay", 64, 16, 8, 256, 700, window=300, seed=5)
+    q, kv = W.generate(w)
+    a, la = _device_run(w, q, kv)
+    w2 = W.Workload("lay", 64, 16, 8, 256, 700, window=300, seed=5, layout="reference")
+    kv2 = np.ascontiguousarray(kv.transpose(2, 0, 1, 3))
+    b, lb = _device_run(w2, q, kv2)
+    assert np.array_equal(a, b) and np.array_equal(la, lb)
+
+
+def test_f16_cache_with_bf16_queries(gpu_ready, po):
+    """The reference's own pairing (bf16 activations, f16 cache) with values outside bf16's grid."""
+    import torch
+    rng = np.random.default_rng(21)
+    c, hq, hkv, hd, kvl = 96, 16, 2, 512, 900
+    q = rng.standard_normal((c, hq, hd)).astype(np.float32)
+    kv = rng.standard_normal((kvl + c, 2, hkv, hd)).astype(np.float32)
+    qb = R.f32_to_bf16_bits_rne(q)
+    kb = R.f32_to_f16_bits_rne(kv)
+    d = A.make_desc(c, hq, hkv, hd, kvl, q_dtype=capi.DG_BF16, kv_dtype=capi.DG_F16, out_dtype=capi.DG_F32)
+    out = torch.zeros(c * hq * hd, dtype=torch.float32, device="cuda")
+    lse = torch.zeros(c * hq, dtype=torch.float32, device="cuda")
+    A.forward(d, A.to_device_bits(qb), A.to_device_bits(kb), out, lse, A.alloc_workspace(d))
+    torch.cuda.synchronize()
+    od = po.make_desc(c, hq, hkv, hd, kvl)
+    ref, ref_lse = po.attention_f32(od, R.bf16_bits_to_f32(qb), R.f16_bits_to_f32(kb))
+    check_tolerances(out.cpu().numpy().reshape(ref.shape), lse.cpu().numpy().reshape(ref_lse.shape), ref, ref_lse,
+                     max_abs=2e-3, mean_abs=1e-4)
+
+
+def test_ring_cache_and_region_offset(gpu_ready, po):
+    """Sliding layer on a wrapped power-of-two ring placed at a non-zero region offset."""
+    import torch
+    rng = np.random.default_rng(31)
+    c, hq, hkv, hd, kvl, window, ring = 256, 16, 8, 256, 5000, 1024, 2048
+    t_all = kvl + c
+    row = 2 * hkv * hd
+    q = rng.standard_normal((c, hq, hd)).astype(np.float32)
+    lin = rng.standard_normal((t_all, row)).astype(np.float32)
+    qb, lb = R.f32_to_bf16_bits_rne(q), R.f32_to_f16_bits_rne(lin)
+    ringbits = np.full((ring, row), 0x7E00, dtype=np.uint16)      # NaN everywhere: dead slots must not be read
+    t_lo = kvl - (window - 1)
+    for pos in range(t_lo, t_all):
+        ringbits[pos & (ring - 1)] = lb[pos]
+    region = 4096
+    buf = np.concatenate([np.full(region // 2, 0x7E00, np.uint16), ringbits.ravel()])
+    d = A.make_desc(c, hq, hkv, hd, kvl, window=window, kv_ring_mask=ring - 1, q_dtype=capi.DG_BF16,
+                    kv_dtype=capi.DG_F16, out_dtype=capi.DG_F32, kv_region_bytes=region)
+    out = torch.zeros(c * hq * hd, dtype=torch.float32, device="cuda")
+    lse = torch.zeros(c * hq, dtype=torch.float32, device="cuda")
+    A.forward(d, A.to_device_bits(qb), A.to_device_bits(buf), out, lse, A.alloc_workspace(d))
+    torch.cuda.synchronize()
+    od = po.make_desc(c, hq, hkv, hd, kvl, window=window)
+    ref, ref_lse = po.attention_f32(od, R.bf16_bits_to_f32(qb), R.f16_bits_to_f32(lb))
+    check_tolerances(out.cpu().numpy().reshape(ref.shape), lse.cpu().numpy().reshape(ref_lse.shape), ref, ref_lse,
+                     max_abs=2e-3, mean_abs=1e-4)
+
+
+def test_truncating_store_matches_reference_rounding(gpu_ready):
+    import torch
+    f = A.model_full_fixture(300, canvas=32)
+    rig = A.AttnRig.from_fixture(f)
+    d32 = rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=False)
+    d32.out_dtype = capi.DG_F32
+    out32 = torch.zeros(f.out_len(), dtype=torch.float32, device="cuda")
+    A.forward(d32, rig.buf_q, rig.buf_kv, out32, rig.buf_lse, rig.workspace_for(d32))
+    rig.run_forward(rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=True))
+    trunc = rig.read_out_f32()
+    rig.run_forward(rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=False))
+    rne = rig.read_out_f32()
+    full = out32.cpu().numpy()
+    assert np.array_equal(trunc, R.bf16_bits_to_f32(R.f32_to_bf16_bits_trunc(full)))
+    assert np.array_equal(rne, R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(full)))
+
+
+def test_row_without_visible_keys(gpu_ready):
+    """An empty key range stores zeros and LSE = -inf instead of NaN (attention_mma2.metal:297)."""
+    import torch
+    w = W.Workload("empty", 16, 4, 2, 64, 40, t_lo=56, seed=1)   # t_lo == t_all
+    for kernel in (capi.DG_KERNEL_MFMA, capi.DG_KERNEL_SCALAR):
+        q, kv = W.generate(w)
+        qd, kd = W.device_arrays(w, q, kv)
+        d = w.desc(kernel=kernel)
+        out = torch.full((w.canvas * w.n_q_heads * w.head_dim,), 7, dtype=torch.int16, device="cuda")
+        lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+        A.forward(d, qd, kd, out, lse, A.alloc_workspace(d))
+        torch.cuda.synchronize()
+        assert torch.all(out == 0) and torch.all(torch.isneginf(lse))
+
+
+def test_runtime_error_codes(gpu_ready):
+    import torch
+    w = W.scaled(W.config("cfg3_global"), 4096)
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+    d = w.desc()
+    out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.int16, device="cuda")
+    lib = capi.load()
+    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    rc = lib.dg_attn_forward(C.byref(d), qd.data_ptr(), kd.data_ptr(), out.data_ptr(), None, small.data_ptr(), 1024,
+                             A.stream_handle())
+    assert rc == capi.DG_ERR_WORKSPACE
+    rc = lib.dg_attn_forward(C.byref(d), qd.data_ptr(), kd.data_ptr(), out.data_ptr(), None, None, 0, A.stream_handle())
+    assert rc == capi.DG_ERR_WORKSPACE
+    rc = lib.dg_attn_forward(C.byref(d), qd.data_ptr() + 2, kd.data_ptr(), out.data_ptr(), None, small.data_ptr(),
+                             1 << 30, A.stream_handle())
+    assert rc == capi.DG_ERR_LAYOUT
+    with pytest.raises(capi.DgAttnError):
+        A.forward(W.Workload("bad", 8, 4, 2, 96, 8).desc(), qd, kd, out)
+    torch.cuda.synchronize()
+
+
+def test_hip_graph_replay(gpu_ready):
+    """The call is capturable: no allocation, no host sync, no memset nodes.  Replays with
+    eager work in between must keep matching the eager result."""
+    import torch
+    w = W.scaled(W.config("cfg3_global"), 4096)
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+    d = w.desc()
+    n = w.canvas * w.n_q_heads * w.head_dim
+    out_e = torch.zeros(n, dtype=torch.int16, device="cuda")
+    out_g = torch.zeros(n, dtype=torch.int16, device="cuda")
+    ws = A.alloc_workspace(d)
+    A.forward(d, qd, kd, out_e, None, ws)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        A.forward(d, qd, kd, out_g, None, ws)     # warm the side stream
+    torch.cuda.current_stream().wait_stream(s)
+    with torch.cuda.graph(g):
+        A.forward(d, qd, kd, out_g, None, ws)
+    for i in range(4):
+        out_g.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), i
+        A.forward(d, qd, kd, out_e, None, ws)     # eager work between replays
+        torch.cuda.synchronize()

@@ -1,0 +1,157 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the
+header declares, the reference-shaped structs have the reference's sizes, descriptor
+validation returns the documented status codes, and the KV layout arithmetic matches the
+reference's (src/metal/step_kv/mod.rs:65-100, src/metal/step_kernel/mod.rs:511-587)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from diffgemma_amd import attention as A
+from diffgemma_amd import capi, step_kv, workloads as W
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "dg_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.load()
+    names = header_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/dg_attn.h but not exported"
+    assert set(names) == set(capi.EXPORTS)
+    assert lib.dg_attn_abi_version() == 1
+
+
+def test_reference_struct_sizes():
+    assert C.sizeof(capi.LayerOffsets) == 200     # 23 u64 + 4 u32, repr(C)
+    assert C.sizeof(capi.StepParams) == 48
+    assert C.sizeof(capi.AttnDims) == 16
+    assert C.sizeof(capi.AttnBlockRange) == 16
+    assert C.sizeof(capi.DebugStatus) == 16
+    assert capi.LayerOffsets.kv_region.offset == 176 and capi.LayerOffsets.kv_ring_mask.offset == 196
+    assert C.sizeof(capi.AttnDesc) == 112
+
+
+def test_strerror_covers_every_status():
+    seen = set()
+    for code in range(0, -10, -1):
+        text = capi.strerror(code)
+        assert text and text != "unknown status"
+        seen.add(text)
+    assert len(seen) == 10
+    assert capi.strerror(-99) == "unknown status"
+
+
+def _status(desc):
+    n = C.c_size_t(0)
+    return capi.load().dg_attn_workspace_bytes(C.byref(desc), C.byref(n))
+
+
+def test_descriptor_validation_codes():
+    ok = A.make_desc(256, 16, 2, 512, 1024)
+    assert _status(ok) == capi.DG_OK
+    assert _status(A.make_desc(256, 16, 2, 96, 1024)) == capi.DG_ERR_SHAPE         # head_dim
+    assert _status(A.make_desc(0, 16, 2, 512, 1024)) == capi.DG_ERR_SHAPE          # empty canvas
+    assert _status(A.make_desc(256, 16, 3, 512, 1024)) == capi.DG_ERR_SHAPE        # Hq % Hkv
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, causal_rows=257)) == capi.DG_ERR_MASK
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_ring_mask=1000)) == capi.DG_ERR_LAYOUT
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_ring_mask=15)) == capi.DG_ERR_LAYOUT  # ring < key tile
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_dtype=7)) == capi.DG_ERR_DTYPE
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, q_dtype=capi.DG_F16, kv_dtype=capi.DG_BF16)) == capi.DG_ERR_DTYPE
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, out_dtype=capi.DG_F16)) == capi.DG_ERR_DTYPE
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, kernel=9)) == capi.DG_ERR_UNSUPPORTED
+    assert _status(A.make_desc(256, 16, 2, 512, 1024, flags=capi.DG_ATTN_F_T_LO_EXPLICIT, t_lo=5000)) == capi.DG_ERR_MASK
+    bad = A.make_desc(256, 16, 2, 512, 1024)
+    bad.k_tok_stride = 1028                                                        # not 16-byte rows
+    assert _status(bad) == capi.DG_ERR_LAYOUT
+    bad = A.make_desc(256, 16, 2, 512, 1024)
+    bad.kv_region_bytes = 8
+    assert _status(bad) == capi.DG_ERR_LAYOUT
+    assert capi.load().dg_attn_workspace_bytes(None, None) == capi.DG_ERR_NULL
+
+
+def test_forward_rejects_null_pointers_before_touching_a_device():
+    d = A.make_desc(4, 4, 2, 32, 8)
+    assert capi.load().dg_attn_forward(C.byref(d), None, None, None, None, None, 0, None) == capi.DG_ERR_NULL
+    assert capi.load().dg_attention_dispatch(None, None, None, None, None, None, None, None, 0, None) == capi.DG_ERR_NULL
+
+
+def test_layout_helpers():
+    d = A.make_desc(256, 16, 8, 256, 4096, layout="reference")
+    assert (d.k_tok_stride, d.k_head_stride, d.v_base_off, d.v_tok_stride, d.v_head_stride) == (4096, 256, 2048, 4096, 256)
+    d = A.make_desc(256, 16, 2, 512, 32768, layout="head_major")
+    t = 32768 + 256
+    assert (d.k_tok_stride, d.k_head_stride, d.v_base_off, d.v_tok_stride, d.v_head_stride) == (512, t * 512, 2 * t * 512, 512, t * 512)
+
+
+def test_split_planning():
+    assert capi.resolved_splits(W.config("cfg3_global").desc()) == 8          # 32 (tile, head) pairs x 8 = 256 workgroups
+    assert capi.resolved_splits(W.config("cfg4_long").desc()) == 8
+    assert capi.resolved_splits(W.config("cfg2_sliding").desc()) == 8
+    assert capi.resolved_splits(A.make_desc(2, 4, 2, 32, 2)) == 1                 # one tile: nothing to split
+    assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, n_splits=3)) == 3
+    assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, kernel=capi.DG_KERNEL_SCALAR)) == 1
+    # workspace: 8 splits x 2 heads x 2048 rows x (512 + 2) floats
+    assert capi.workspace_bytes(W.config("cfg3_global").desc()) == 8 * 2 * 2048 * 514 * 4
+    assert capi.workspace_bytes(A.make_desc(2, 4, 2, 32, 2)) == 0
+
+
+def test_visible_pairs_and_flops():
+    pairs, flops = capi.visible_pairs(W.config("cfg3_global").desc())
+    assert pairs == 8429632 and flops == 4.0 * 512 * 16 * 8429632
+    assert capi.visible_pairs(W.config("cfg3_global_b").desc())[0] == 8446016
+    assert capi.visible_pairs(W.config("cfg2_sliding").desc())[0] == 256 * 1279
+    assert capi.visible_pairs(W.config("cfg2_sliding_768").desc())[0] == 256 * 1024
+    assert capi.visible_pairs(W.config("cfg4_long").desc())[0] == 256 * 131328
+
+
+def test_host_and_oracle_agree_on_pair_counts(po):
+    import itertools
+    lib = po.load()
+    for c, kvl, cr, win, sees in itertools.product((1, 7, 64), (0, 5, 300), (0, 3, 64), (0, 2, 50), (0, 1)):
+        if cr > c:
+            continue
+        d = A.make_desc(c, 4, 2, 32, kvl, causal_rows=cr, window=win,
+                        flags=capi.DG_ATTN_F_CAUSAL_SEES_MASKED if sees else 0)
+        od = po.make_desc(c, 4, 2, 32, kvl, causal_rows=cr, window=win, causal_sees_masked=sees)
+        assert capi.visible_pairs(d)[0] == lib.dgo_visible_pairs(C.byref(od)), (c, kvl, cr, win, sees)
+
+
+def test_kv_layout_arithmetic():
+    assert step_kv.kv_row_bytes(256) == 512 and step_kv.kv_row_bytes(512) == 1024
+    assert step_kv.kv_region_bytes(8, 256, 4096) == 4096 * 8 * 2 * 512          # 32 MiB ring
+    assert step_kv.layer_kv_slots(True, 32768 + 256) == 33032                   # (max_seq + 8) rounded to 8
+    assert step_kv.layer_kv_slots(False, 33024) == 4096                         # pow2 capped at the ring size
+    assert step_kv.layer_kv_slots(False, 1000) == 1024
+    assert step_kv.kv_slot(4095, 5000) == 5000 & 4095 and step_kv.kv_slot(0, 5000) == 5000
+    layers = step_kv.build_layout(33024)
+    assert [l.layer for l in layers if l.is_full] == [5, 11, 17, 23, 29]
+    assert layers[0].kv_region == 0 and layers[1].kv_region == 32 << 20
+    assert layers[6].kv_region == 6 * (32 << 20) - (32 << 20) + step_kv.kv_region_bytes(2, 512, 33032)
+    assert all(l.kv_ring_mask == (0 if l.is_full else 4095) for l in layers)
+    total = step_kv.kv_cache_total_bytes(layers)
+    assert total == 25 * (32 << 20) + 5 * step_kv.kv_region_bytes(2, 512, 33032)
+    lo = layers[5].offsets()
+    assert (lo.head_dim, lo.n_kv_heads, lo.is_full, lo.kv_ring_mask) == (512, 2, 1, 0)
+
+
+def test_profile_helpers_refuse_misuse():
+    lib = capi.load()
+    assert lib.dg_prof_end(None, None) == capi.DG_ERR_UNSUPPORTED   # not begun
+
+
+def test_workload_table():
+    w = W.config("cfg3_global")
+    assert (w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, w.causal_rows) == (256, 16, 2, 512, 32768, 128)
+    w = W.scaled(W.config("cfg2_sliding_768"), 2048)
+    assert w.t_lo == 2048 - 768
+    with pytest.raises(KeyError):
+        W.config("nope")
