@@ -37,6 +37,26 @@ typedef __attribute__((address_space(3))) void lds_void;
 
 constexpr float kTau = 8.0f;  // log2 units: P never exceeds 2^8 before a rescale
 
+// Optional per-phase cycle accounting (development builds only): every wave sums the cycles
+// it spends in each phase of the tile loop and stores the sums at the end.
+#ifdef DG_ATTN_PHASE_TIMING
+#define DG_PHASE_DECL unsigned long long ph_t = clock64(), ph_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define DG_PHASE(i)                          \
+  {                                          \
+    const unsigned long long now = clock64(); \
+    ph_acc[i] += now - ph_t;                 \
+    ph_t = now;                              \
+  }
+#define DG_PHASE_STORE                                                                    \
+  if (p.phase_cycles && lane == 0) {                                                      \
+    for (int i = 0; i < 8; ++i) p.phase_cycles[((size_t)blockIdx.x * 4 + wave) * 8 + i] = ph_acc[i]; \
+  }
+#else
+#define DG_PHASE_DECL
+#define DG_PHASE(i)
+#define DG_PHASE_STORE
+#endif
+
 template <bool F16>
 __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
   if constexpr (F16) {
@@ -72,6 +92,14 @@ __device__ __forceinline__ float unpack_hi(uint32_t u) {
   else return __uint_as_float(u & 0xffff0000u);
 }
 
+// s_waitcnt vmcnt(0) as a builtin, so that the compiler's own wait-count bookkeeping sees it
+// (gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt = 6:4, lgkmcnt = 11:8; the other two
+// counters are left at their maxima).
+__device__ __forceinline__ void wait_vmem_all() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
+}
+
 // value of lane l combined with lane l^32
 __device__ __forceinline__ float max_across_halves(float x) {
   const uint32_t u = __float_as_uint(x);
@@ -97,29 +125,60 @@ __device__ __forceinline__ uint32_t swz_v(uint32_t row) {
   return ((row & 3u) << 2) & (CPR - 1);
 }
 
-// Queue the direct-to-LDS loads of one 32-key tile.  Each wave instruction fills one
-// contiguous KiB of LDS (64 lanes x 16 B); the swizzle is applied by choosing which global
-// chunk each lane fetches.  Keys past t_all re-read key t_all-1 (finite data, masked later).
+// One 32-key tile's direct-to-LDS loads, described once per tile and issued one wave
+// instruction at a time so the issue slots can be spread between MFMAs.  Each instruction
+// fills one contiguous KiB of LDS (64 lanes x 16 B); the swizzle is applied by choosing which
+// global chunk each lane fetches.  Keys past t_all re-read key t_all-1 (finite, masked later).
+struct TileLoad {
+  const char* base;   // head base + slot(t0) * row stride (wave-uniform)
+  uint32_t stride_b;  // bytes between key rows
+  uint32_t rmax;      // last valid row of the tile
+  uint32_t lds;       // LDS byte address of the destination buffer
+  bool on;
+};
+
+__device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_t tok_stride_b, uint32_t t0,
+                                                   uint32_t t_all, uint32_t ring_mask, lds_char* buf, bool on) {
+  TileLoad tl;
+  tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
+  tl.stride_b = (uint32_t)tok_stride_b;
+  tl.rmax = t_all - 1u - t0;
+  tl.lds = (uint32_t)(size_t)buf;
+  tl.on = on;
+  return tl;
+}
+
+// The load is written as assembly on purpose: the compiler orders every LDS read after a
+// direct-to-LDS load it knows about with s_waitcnt vmcnt(0), which would expose the whole
+// fetch latency once per tile.  The kernel waits for these loads itself, at the top of the
+// tile loop, one iteration after they were issued.
 template <int D, bool IS_V>
-__device__ __forceinline__ void issue_tile(const char* head_base, int64_t tok_stride_b, uint32_t t0,
-                                           uint32_t t_all, uint32_t ring_mask, lds_char* buf, uint32_t wave,
-                                           uint32_t lane) {
+__device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint32_t wave, uint32_t lane) {
   constexpr int CPR = D / 8;
   constexpr int NBLK = 32 * CPR / 64;
-  const uint32_t slot0 = kv_slot(ring_mask, t0);
-  const char* base = head_base + (int64_t)slot0 * tok_stride_b;
-  const uint32_t rmax = t_all - 1u - t0;
+  if (!tl.on) return;
+  const uint32_t blk = k * 4 + wave;
+  if (NBLK < 4 && blk >= (uint32_t)NBLK) return;
+  const uint32_t pch = blk * 64 + lane;
+  const uint32_t r = pch / CPR, pc = pch % CPR;
+  const uint32_t c = pc ^ (IS_V ? swz_v<CPR>(r) : swz_k<CPR>(r));
+  const uint32_t voff = min(r, tl.rmax) * tl.stride_b + c * 16u;
+  // both are wave-uniform by construction; readfirstlane tells the compiler so
+  const uint32_t dst = __builtin_amdgcn_readfirstlane(tl.lds + blk * 1024u);
+  const uint64_t b = (uint64_t)tl.base;
+  // (readfirstlane returns a signed int: without the casts the low half would be sign-extended
+  // over the high half)
+  const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32) |
+                        (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base)
+               : "memory");
+}
+
+template <int D, bool IS_V>
+__device__ __forceinline__ void issue_tile(const TileLoad& tl, uint32_t wave, uint32_t lane) {
+  constexpr int NLD = (32 * (D / 8) / 64 + 3) / 4;
 #pragma unroll
-  for (int k = 0; k < (NBLK + 3) / 4; ++k) {
-    const uint32_t blk = k * 4 + wave;
-    if (NBLK < 4 && blk >= (uint32_t)NBLK) continue;
-    const uint32_t pch = blk * 64 + lane;
-    const uint32_t r = pch / CPR, pc = pch % CPR;
-    const uint32_t c = pc ^ (IS_V ? swz_v<CPR>(r) : swz_k<CPR>(r));
-    const uint32_t reff = min(r, rmax);
-    const uint32_t voff = reff * (uint32_t)tok_stride_b + c * 16u;
-    __builtin_amdgcn_global_load_lds((gbl_void*)(base + voff), (lds_void*)(buf + blk * 1024), 16, 0, 0);
-  }
+  for (int k = 0; k < NLD; ++k) issue_tile_part<D, IS_V>(tl, k, wave, lane);
 }
 
 // PIPE: issue Q.K^T of tile j+1 before the softmax of tile j (needs a second score tile in
@@ -226,32 +285,67 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const uint32_t v_lane_chunk = 2u * h16 + ((i16 & 3u) >> 1);
   const uint32_t v_lane_off = v_row * ROWB + (i16 & 1u) * 8u;
 
-  auto qk_tile = [&](lds_char* kb) -> f32x16 {
+  constexpr int NLD = (32 * CPR / 64 + 3) / 4;   // load instructions per wave, tile and matrix
+  constexpr int NQK = NSTEP, NPV = 2 * NDB;      // MFMAs per tile in each phase
+  constexpr int PFK = NQK < 4 ? NQK : 4;         // fragment reads kept in flight ahead of the MFMAs
+  constexpr int PFV = NPV < 4 ? NPV : 4;
+  constexpr int LDK_EVERY = NQK / NLD, LDV_EVERY = NPV / NLD;
+
+  auto k_frag = [&](lds_char* kb, int st) -> u32x4 {
+    const uint32_t c = (uint32_t)(2 * st) + g2;
+    return *(lds_u32x4*)(kb + k_row_off + ((c ^ k_swz) << 4));
+  };
+  auto v_frag = [&](lds_char* vb, int i) -> u32x4 {   // i = ks * NDB + db
+    const int ks = i / NDB, db = i % NDB;
+    const uint32_t c = (uint32_t)(4 * db) + v_lane_chunk;
+    const uint32_t off = v_lane_off + (uint32_t)(16 * ks) * ROWB + ((c ^ v_swz) << 4);
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off)));
+    const u32x2 hi =
+        __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off + 8 * ROWB)));
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+  };
+
+  // S^T = K.Q^T for one tile.  PFK fragment reads run ahead of the MFMA that consumes them and
+  // the next K tile's global loads are issued one instruction every LDK_EVERY MFMAs; the
+  // scheduling barriers keep that interleaving.
+  auto qk_tile = [&](lds_char* kb, const TileLoad& next_k, uint32_t ld_lane) -> f32x16 {
     f32x16 s;
 #pragma unroll
     for (int e = 0; e < 16; ++e) s[e] = 0.f;
+    u32x4 kf[PFK];
 #pragma unroll
-    for (int st = 0; st < NSTEP; ++st) {
-      const uint32_t c = (uint32_t)(2 * st) + g2;
-      const u32x4 a = *(lds_u32x4*)(kb + k_row_off + ((c ^ k_swz) << 4));
-      s = mfma16<F16>(a, qf[st], s);
+    for (int i = 0; i < PFK; ++i) kf[i] = k_frag(kb, i);
+#pragma unroll
+    for (int st = 0; st < NQK; ++st) {
+      __builtin_amdgcn_sched_barrier(0);
+      s = mfma16<F16>(kf[st % PFK], qf[st], s);
+      if (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
+      if (st % LDK_EVERY == 0 && st / LDK_EVERY < NLD) issue_tile_part<D, false>(next_k, st / LDK_EVERY, wave, ld_lane);
     }
+    __builtin_amdgcn_sched_barrier(0);
     return s;
   };
 
+  DG_PHASE_DECL
   if (ntile > 0) {
     lds_char* const k0 = (lds_char*)sk0;
     lds_char* const k1 = (lds_char*)sk1;
     lds_char* const v0 = (lds_char*)sv0;
     lds_char* const v1 = (lds_char*)sv1;
+    const TileLoad none = make_tile_load(kbase, kstride_b, tb * kBlockN, p.t_all, p.ring_mask, k0, false);
 
-    issue_tile<D, false>(kbase, kstride_b, tb * kBlockN, p.t_all, p.ring_mask, k0, wave, lane);
-    if (ntile > 1) issue_tile<D, false>(kbase, kstride_b, (tb + 1) * kBlockN, p.t_all, p.ring_mask, k1, wave, lane);
-    issue_tile<D, true>(vbase, vstride_b, tb * kBlockN, p.t_all, p.ring_mask, v0, wave, lane);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    issue_tile<D, false>(make_tile_load(kbase, kstride_b, tb * kBlockN, p.t_all, p.ring_mask, k0, true), wave, lane);
+    if (ntile > 1)
+      issue_tile<D, false>(make_tile_load(kbase, kstride_b, (tb + 1) * kBlockN, p.t_all, p.ring_mask, k1, true), wave, lane);
+    issue_tile<D, true>(make_tile_load(vbase, vstride_b, tb * kBlockN, p.t_all, p.ring_mask, v0, true), wave, lane);
+    wait_vmem_all();
     __syncthreads();
     f32x16 s_cur;
-    if constexpr (PIPE) s_cur = qk_tile(k0);
+    if constexpr (PIPE) {
+      // K(tb+2) goes where K(tb) sits, so it cannot be issued before this first tile is consumed
+      s_cur = qk_tile(k0, none, lane);
+    }
+    DG_PHASE(0)
 
     for (uint32_t jj = 0; jj < ntile; ++jj) {
       const uint32_t t0 = (tb + jj) * kBlockN;
@@ -261,24 +355,34 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       lds_char* const vb_free = (jj & 1u) ? v0 : v1;   // refill with V(jj+1)
 
       // The tiles this iteration reads have landed everywhere, and every wave is done with
-      // the buffers about to be refilled.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // the buffers this iteration refills.
+      wait_vmem_all();
+      DG_PHASE(1)
       __syncthreads();
-      if constexpr (PIPE) {
-        // K(jj) was consumed one iteration ago: its buffer takes K(jj+2)
-        if (jj + 2 < ntile) issue_tile<D, false>(kbase, kstride_b, t0 + 2 * kBlockN, p.t_all, p.ring_mask, kb_even, wave, lane);
-      } else {
-        // K(jj+1) goes to the other buffer (prologue loaded K(tb+1) already for jj == 0)
-        if (jj >= 1 && jj + 1 < ntile) issue_tile<D, false>(kbase, kstride_b, t0 + kBlockN, p.t_all, p.ring_mask, kb_odd, wave, lane);
-      }
-      if (jj + 1 < ntile) issue_tile<D, true>(vbase, vstride_b, t0 + kBlockN, p.t_all, p.ring_mask, vb_free, wave, lane);
-
+      DG_PHASE(2)
+      // Re-derive the per-lane global offsets of the tile loads inside every iteration: hoisted
+      // out of the loop they would cost sixteen more live VGPRs than this kernel has.
+      uint32_t lane_l = lane;
+      asm volatile("" : "+v"(lane_l));
+      // PIPE: K(jj) was consumed one iteration ago, its buffer takes K(jj+2).
+      // otherwise: K(jj+1) goes to the other buffer (the prologue already fetched K(tb+1)).
+      const TileLoad next_k =
+          PIPE ? make_tile_load(kbase, kstride_b, t0 + 2 * kBlockN, p.t_all, p.ring_mask, kb_even, jj + 2 < ntile)
+               : make_tile_load(kbase, kstride_b, t0 + kBlockN, p.t_all, p.ring_mask, kb_odd,
+                                jj >= 1 && jj + 1 < ntile);
+      const TileLoad next_v =
+          make_tile_load(vbase, vstride_b, t0 + kBlockN, p.t_all, p.ring_mask, vb_free, jj + 1 < ntile);
+      DG_PHASE(3)
       f32x16 s_next;
       if constexpr (PIPE) {
-        if (jj + 1 < ntile) s_next = qk_tile(kb_odd);
+        if (jj + 1 < ntile) s_next = qk_tile(kb_odd, next_k, lane_l);
       } else {
-        s_cur = qk_tile(kb_even);
+        s_cur = qk_tile(kb_even, next_k, lane_l);
       }
+#ifdef DG_ATTN_PHASE_TIMING
+      asm volatile("s_nop 0" ::"v"(s_cur[0]), "v"(s_cur[15]));  // the scores have to exist before the clock is read
+#endif
+      DG_PHASE(4)
 
       // ---- mask (edge tiles only) ----
       const bool masked = !(t0 >= lo_max && t0 + kBlockN <= hi_min);
@@ -326,25 +430,26 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         // the row sum uses the rounded probabilities, the same numbers P.V multiplies
         l_part += unpack_lo<F16>(pk) + unpack_hi<F16>(pk);
       }
+      DG_PHASE(5)
 
-      // ---- O^T += V^T . P^T ----
+      // ---- O^T += V^T . P^T, V(jj+1)'s global loads spread between the MFMAs ----
+      {
+        u32x4 vf[PFV];
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+        for (int i = 0; i < PFV; ++i) vf[i] = v_frag(vb_cur, i);
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const uint32_t c = (uint32_t)(4 * db) + v_lane_chunk;
-          const uint32_t off = v_lane_off + (uint32_t)(16 * ks) * ROWB + ((c ^ v_swz) << 4);
-          const i16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb_cur + off));
-          const i16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb_cur + off + 8 * ROWB));
-          u32x4 a;
-          const u32x2 lo = __builtin_bit_cast(u32x2, a0), hi = __builtin_bit_cast(u32x2, a1);
-          a[0] = lo[0];
-          a[1] = lo[1];
-          a[2] = hi[0];
-          a[3] = hi[1];
-          o[db] = mfma16<F16>(a, pf[ks], o[db]);
+        for (int i = 0; i < NPV; ++i) {
+          __builtin_amdgcn_sched_barrier(0);
+          o[i % NDB] = mfma16<F16>(vf[i % PFV], pf[i / NDB], o[i % NDB]);
+          if (i + PFV < NPV) vf[i % PFV] = v_frag(vb_cur, i + PFV);
+          if (i % LDV_EVERY == 0 && i / LDV_EVERY < NLD) issue_tile_part<D, true>(next_v, i / LDV_EVERY, wave, lane_l);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
+#ifdef DG_ATTN_PHASE_TIMING
+      asm volatile("s_nop 0" ::"a"(o[0][0]), "a"(o[NDB - 1][15]));
+#endif
+      DG_PHASE(6)
       if constexpr (PIPE) {
         if (jj + 1 < ntile) s_cur = s_next;
       }
@@ -352,6 +457,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   }
 
   // ---- epilogue ----
+  DG_PHASE_STORE
   const float l_tot = sum_across_halves(l_part);
   if (p.n_splits > 1) {
     const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + r;

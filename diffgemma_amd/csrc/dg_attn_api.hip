@@ -28,6 +28,10 @@ DeviceInfo g_dev[64];
 thread_local uint32_t* g_tls_dbg = nullptr;
 std::mutex g_dev_mu;
 
+#ifdef DG_ATTN_PHASE_TIMING
+unsigned long long* g_phase_cycles = nullptr;
+#endif
+
 struct ProfState {
   std::vector<hipEvent_t> ev;
   uint32_t used = 0;
@@ -333,6 +337,9 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
     p.part_ml = (float*)(ws + pl.off_part_ml);
   }
   p.dbg = g_tls_dbg;  // set only while dg_attention_dispatch is on the stack
+#ifdef DG_ATTN_PHASE_TIMING
+  p.phase_cycles = g_phase_cycles;
+#endif
 
   if (pl.scalar) {
     if (dg::launch_attn_scalar(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
@@ -387,6 +394,11 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
   g_tls_dbg = nullptr;
   return rc;
 }
+
+#ifdef DG_ATTN_PHASE_TIMING
+// development builds only: device buffer of [workgroups][4][8] cycle sums
+void dg_debug_set_phase_buffer(void* device_ptr) { g_phase_cycles = (unsigned long long*)device_ptr; }
+#endif
 
 int dg_prof_begin(uint32_t max_launches) {
   if (g_prof.active) return DG_ERR_UNSUPPORTED;
