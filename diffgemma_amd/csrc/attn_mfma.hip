@@ -4,18 +4,23 @@
 // Stacked row = canvas_row * group + head_in_group, so the `group` query heads that share a KV
 // head are the M dimension of the same tile and K/V are read once for all of them.
 //
-// Per 32-key tile:
-//   S^T = K . Q^T   v_mfma_f32_32x32x16 (bf16 or f16): A = K rows from LDS (ds_read_b128),
-//                   B = Q held in registers for the whole kernel.  Output lane = query row,
-//                   output registers = keys, so row max / row sum are per-lane scalars.
-//   P   = exp2(S*c - m)  in registers; its register layout already is the B operand of the
-//                   next MFMA when keys are taken in the order the accumulator holds them.
-//   O^T += V^T . P^T  A = V^T fragments read with ds_read_b64_tr_b16 from the row-major V tile.
-// K and V tiles arrive by 16-byte direct-to-LDS loads, double buffered: tile j+2 of K and
-// tile j+1 of V are in flight while tile j+1 of K and tile j of V are consumed.  QK^T of the
-// next tile is issued before the softmax of the current one so the matrix pipe has work
-// while the VALU computes exponentials.  The running max is only raised (and O rescaled)
-// when some row's tile max exceeds it by more than 2^kTau, which in steady state is never.
+// Per 32-key tile every wave plays two roles:
+//   row owner  (32 rows):  S^T = K.Q^T with v_mfma_f32_32x32x16 (bf16 or f16): A = K rows from
+//              LDS (ds_read_b128), B = Q held in registers for the whole kernel.  Output lane =
+//              query row, output registers = keys, so row max / row sum are per-lane scalars.
+//              P = exp2(S*c - m) is rounded to the element type and written to LDS in exactly
+//              the register image the next MFMA wants as its B operand.
+//   d owner (a quarter of head_dim, all 128 rows):  O^T += V^T.P^T, A = V^T fragments read with
+//              ds_read_b64_tr_b16 from the row-major V tile, B = P fragments from LDS.
+// Splitting P.V over head_dim instead of rows is what keeps LDS traffic affordable: the
+// transposing read runs at half the rate of ds_read_b128, and with a row split each of the four
+// waves would read the whole V tile through it; with the d split each V fragment is read once
+// per workgroup and the small P tile is what gets read four times.
+//
+// K and V tiles arrive by 16-byte direct-to-LDS loads, double buffered, issued one instruction
+// at a time between MFMAs.  The running max is only raised (and O rescaled) when some row's
+// tile max exceeds it by more than 2^kTau, which in steady state is never; the raise is
+// broadcast to the d owners through LDS together with P.
 #include "attn_params.h"
 
 namespace dg {
@@ -157,6 +162,9 @@ __device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint3
   constexpr int CPR = D / 8;
   constexpr int NBLK = 32 * CPR / 64;
   if (!tl.on) return;
+#if defined(DG_EXP) && DG_EXP == 1
+  return;   // experiment: no tile loads inside the loop
+#endif
   const uint32_t blk = k * 4 + wave;
   if (NBLK < 4 && blk >= (uint32_t)NBLK) return;
   const uint32_t pch = blk * 64 + lane;
@@ -186,10 +194,19 @@ __device__ __forceinline__ void issue_tile(const TileLoad& tl, uint32_t wave, ui
 template <int D, bool F16, bool PIPE>
 __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   constexpr int CPR = D / 8, ROWB = 2 * D, TILEB = kBlockN * ROWB, NSTEP = D / 16, NDB = D / 32;
+  // P.V work split: DSPLIT groups of d-blocks x RSPLIT groups of row-blocks = 4 waves
+  constexpr int DSPLIT = NDB < 4 ? NDB : 4, RSPLIT = 4 / DSPLIT;
+  constexpr int NDBW = NDB / DSPLIT;   // d-blocks (32 wide) this wave accumulates
+  constexpr int NRBW = 4 / RSPLIT;     // row-blocks (32 rows) this wave accumulates
+  constexpr int NACC = NDBW * NRBW;
   __shared__ __attribute__((aligned(1024))) char sk0[TILEB];
   __shared__ __attribute__((aligned(1024))) char sk1[TILEB];
   __shared__ __attribute__((aligned(1024))) char sv0[TILEB];
   __shared__ __attribute__((aligned(1024))) char sv1[TILEB];
+  __shared__ __attribute__((aligned(1024))) char sp[2 * 4 * 1024];   // P: [ks][row-block][lane] x 16 B
+  __shared__ __attribute__((aligned(16))) float scorr[4 * 32];       // per-row rescale factor of this tile
+  __shared__ __attribute__((aligned(16))) uint32_t sflag[4];         // row-block raised its max this tile
+  __shared__ __attribute__((aligned(16))) float sml[4 * 32 * 2];     // epilogue: (m, l) per row
 
   // ---- which (KV head, split, row tile) this workgroup owns ----
   // Workgroup ids go round-robin over the 8 XCDs.  All row tiles of one (KV head, split)
@@ -205,8 +222,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t g2 = lane >> 5, l32 = lane & 31u, h16 = (lane >> 4) & 1u, i16 = lane & 15u;
+  const uint32_t dgrp = wave % DSPLIT, rgrp = wave / DSPLIT;
 
-  // ---- this lane's query row and its key bounds ----
+  // ---- row-owner role: this lane's query row and its key bounds ----
   const uint32_t row0 = mt * kBlockM;
   const uint32_t r = row0 + wave * 32u + l32;
   const bool row_ok = r < p.rows_total;
@@ -265,9 +283,11 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     }
   }
 
-  f32x16 o[NDB];
+  // d-owner accumulators: o[i * NRBW + j] = O^T block (d-block dgrp*NDBW+i, row-block rgrp*NRBW+j);
+  // register e of a block is d offset 8*(e>>2) + 4*g2 + (e&3), the lane is the row (l32).
+  f32x16 o[NACC];
 #pragma unroll
-  for (int i = 0; i < NDB; ++i)
+  for (int i = 0; i < NACC; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[i][e] = 0.f;
   float m_ref = -INFINITY;  // running reference max, log2 units (scale folded in)
@@ -284,25 +304,29 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const uint32_t v_swz = swz_v<CPR>(v_row);
   const uint32_t v_lane_chunk = 2u * h16 + ((i16 & 3u) >> 1);
   const uint32_t v_lane_off = v_row * ROWB + (i16 & 1u) * 8u;
+  lds_char* const pbuf = (lds_char*)sp;
 
   constexpr int NLD = (32 * CPR / 64 + 3) / 4;   // load instructions per wave, tile and matrix
-  constexpr int NQK = NSTEP, NPV = 2 * NDB;      // MFMAs per tile in each phase
-  constexpr int PFK = NQK < 4 ? NQK : 4;         // fragment reads kept in flight ahead of the MFMAs
-  constexpr int PFV = NPV < 4 ? NPV : 4;
+  constexpr int NQK = NSTEP, NPV = 2 * NACC;     // MFMAs per wave and tile in each phase
+  constexpr int PFK = NQK < 4 ? NQK : 4;         // K fragment reads kept in flight ahead of the MFMAs
   constexpr int LDK_EVERY = NQK / NLD, LDV_EVERY = NPV / NLD;
 
   auto k_frag = [&](lds_char* kb, int st) -> u32x4 {
     const uint32_t c = (uint32_t)(2 * st) + g2;
     return *(lds_u32x4*)(kb + k_row_off + ((c ^ k_swz) << 4));
   };
-  auto v_frag = [&](lds_char* vb, int i) -> u32x4 {   // i = ks * NDB + db
-    const int ks = i / NDB, db = i % NDB;
-    const uint32_t c = (uint32_t)(4 * db) + v_lane_chunk;
+  // V^T fragment for MFMA k-step ks of d-block db: k-slot j of lane half g2 is key
+  // 16*ks + 8*(j>>2) + 4*g2 + (j&3), the order in which the score accumulator holds keys.
+  auto v_frag = [&](lds_char* vb, int ks, uint32_t db) -> u32x4 {
+    const uint32_t c = 4u * db + v_lane_chunk;
     const uint32_t off = v_lane_off + (uint32_t)(16 * ks) * ROWB + ((c ^ v_swz) << 4);
     const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off)));
     const u32x2 hi =
         __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off + 8 * ROWB)));
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
+  };
+  auto p_frag = [&](int ks, uint32_t rbk) -> u32x4 {
+    return *(lds_u32x4*)(pbuf + (((uint32_t)ks * 4u + rbk) * 64u + lane) * 16u);
   };
 
   // S^T = K.Q^T for one tile.  PFK fragment reads run ahead of the MFMA that consumes them and
@@ -320,7 +344,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       __builtin_amdgcn_sched_barrier(0);
       s = mfma16<F16>(kf[st % PFK], qf[st], s);
       if (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
+#if !defined(DG_EXP) || DG_EXP != 3
       if (st % LDK_EVERY == 0 && st / LDK_EVERY < NLD) issue_tile_part<D, false>(next_k, st / LDK_EVERY, wave, ld_lane);
+#endif
     }
     __builtin_amdgcn_sched_barrier(0);
     return s;
@@ -354,8 +380,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       lds_char* const vb_cur = (jj & 1u) ? v1 : v0;    // holds V(jj)
       lds_char* const vb_free = (jj & 1u) ? v0 : v1;   // refill with V(jj+1)
 
-      // The tiles this iteration reads have landed everywhere, and every wave is done with
-      // the buffers this iteration refills.
+      // Barrier A: the tiles this iteration reads have landed everywhere, and every wave is done
+      // with the previous tile (its K/V buffers, the P tile and the rescale words can be reused).
       wait_vmem_all();
       DG_PHASE(1)
       __syncthreads();
@@ -372,7 +398,10 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
                                 jj >= 1 && jj + 1 < ntile);
       const TileLoad next_v =
           make_tile_load(vbase, vstride_b, t0 + kBlockN, p.t_all, p.ring_mask, vb_free, jj + 1 < ntile);
-      DG_PHASE(3)
+#if defined(DG_EXP) && DG_EXP == 3
+      issue_tile<D, false>(next_k, wave, lane_l);
+      issue_tile<D, true>(next_v, wave, lane_l);
+#endif
       f32x16 s_next;
       if constexpr (PIPE) {
         if (jj + 1 < ntile) s_next = qk_tile(kb_odd, next_k, lane_l);
@@ -382,7 +411,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #ifdef DG_ATTN_PHASE_TIMING
       asm volatile("s_nop 0" ::"v"(s_cur[0]), "v"(s_cur[15]));  // the scores have to exist before the clock is read
 #endif
-      DG_PHASE(4)
+      DG_PHASE(3)
 
       // ---- mask (edge tiles only) ----
       const bool masked = !(t0 >= lo_max && t0 + kBlockN <= hi_min);
@@ -398,56 +427,95 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
       for (int e = 1; e < 16; ++e) tmax = fmaxf(tmax, s_cur[e]);
       tmax = max_across_halves(tmax) * p.scale_log2;
-      if (__builtin_amdgcn_ballot_w64(tmax > m_ref + kTau) != 0ull) {
+      const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau) != 0ull;
+      if (raise) {
         const float m_new = fmaxf(m_ref, tmax);
         const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
         l_part *= corr;
-        // O lives in accumulator registers, which only MFMA and the accvgpr moves can touch.
-        // Spelling the multiply out keeps the values in that register class on both sides
-        // of this rarely taken branch; a plain `o[i] *= corr` makes the allocator shuttle
-        // all of O through VGPRs and spill.
-#pragma unroll
-        for (int i = 0; i < NDB; ++i)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            float tmp;
-            float x = o[i][e];
-            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
-                         : "+a"(x), "=&v"(tmp)
-                         : "v"(corr));
-            o[i][e] = x;
-          }
+        if (g2 == 0) scorr[wave * 32u + l32] = corr;   // the d owners rescale O after barrier B
         m_ref = m_new;
       }
+      if (lane == 0) sflag[wave] = raise ? 1u : 0u;
       const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
-      u32x4 pf[2];
 #pragma unroll
-      for (int e = 0; e < 16; e += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e], p.scale_log2, -m_use));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e + 1], p.scale_log2, -m_use));
-        const uint32_t pk = pack2<F16>(p0, p1);
-        pf[e >> 3][(e >> 1) & 3] = pk;
-        // the row sum uses the rounded probabilities, the same numbers P.V multiplies
-        l_part += unpack_lo<F16>(pk) + unpack_hi<F16>(pk);
+      for (int ks = 0; ks < 2; ++ks) {
+        u32x4 pk4;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          const int e = 8 * ks + j;
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e], p.scale_log2, -m_use));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e + 1], p.scale_log2, -m_use));
+          const uint32_t pk = pack2<F16>(p0, p1);
+          pk4[j >> 1] = pk;
+          // the row sum uses the rounded probabilities, the same numbers P.V multiplies
+          l_part += unpack_lo<F16>(pk) + unpack_hi<F16>(pk);
+        }
+        // register image of the B operand of MFMA k-step ks for (row l32, lane half g2)
+        *(lds_u32x4*)(pbuf + (((uint32_t)ks * 4u + wave) * 64u + lane) * 16u) = pk4;
       }
+      DG_PHASE(4)
+      // Barrier B: P and the rescale words of this tile are visible to the d owners.
+      __syncthreads();
       DG_PHASE(5)
 
-      // ---- O^T += V^T . P^T, V(jj+1)'s global loads spread between the MFMAs ----
+      // ---- d-owner role ----
       {
-        u32x4 vf[PFV];
+        const u32x4 fl = *(lds_u32x4*)((lds_char*)sflag);
+        if (__builtin_amdgcn_readfirstlane(fl[0] | fl[1] | fl[2] | fl[3]) != 0u) {
+          // O lives in accumulator registers, which only MFMA and the accvgpr moves can touch.
+          // Spelling the multiply out keeps the values in that register class on both sides of
+          // this rarely taken branch; a plain `o[i] *= corr` makes the allocator shuttle all of
+          // O through VGPRs and spill.
 #pragma unroll
-        for (int i = 0; i < PFV; ++i) vf[i] = v_frag(vb_cur, i);
+          for (int j = 0; j < NRBW; ++j) {
+            const uint32_t rbk = rgrp * NRBW + j;
+            if (__builtin_amdgcn_readfirstlane(fl[rbk]) == 0u) continue;
+            const float corr = scorr[rbk * 32u + l32];
 #pragma unroll
-        for (int i = 0; i < NPV; ++i) {
-          __builtin_amdgcn_sched_barrier(0);
-          o[i % NDB] = mfma16<F16>(vf[i % PFV], pf[i / NDB], o[i % NDB]);
-          if (i + PFV < NPV) vf[i % PFV] = v_frag(vb_cur, i + PFV);
-          if (i % LDV_EVERY == 0 && i / LDV_EVERY < NLD) issue_tile_part<D, true>(next_v, i / LDV_EVERY, wave, lane_l);
+            for (int i = 0; i < NDBW; ++i)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                float tmp;
+                float x = o[i * NRBW + j][e];
+                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                             : "+a"(x), "=&v"(tmp)
+                             : "v"(corr));
+                o[i * NRBW + j][e] = x;
+              }
+          }
+        }
+        // O^T += V^T . P^T: per k-step, NDBW V^T fragments x NRBW P fragments.  The P fragments
+        // of a k-step stay in registers for the whole step; the V^T fragment of the next d-block
+        // is fetched while the current one multiplies, and each P fragment of k-step 1 replaces
+        // its k-step 0 counterpart right after that one's last use.  V(jj+1)'s global loads are
+        // spread between the MFMAs.
+        u32x4 pbv[NRBW];
+#pragma unroll
+        for (int j = 0; j < NRBW; ++j) pbv[j] = p_frag(0, rgrp * NRBW + j);
+        u32x4 va_cur = v_frag(vb_cur, 0, dgrp * NDBW), va_next = va_cur;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+          for (int i = 0; i < NDBW; ++i) {
+            const int nxt = ks * NDBW + i + 1;   // next (k-step, d-block) pair
+            if (nxt < 2 * NDBW) va_next = v_frag(vb_cur, nxt / NDBW, dgrp * NDBW + nxt % NDBW);
+#pragma unroll
+            for (int j = 0; j < NRBW; ++j) {
+              const int n = (ks * NDBW + i) * NRBW + j;   // MFMA index within the tile
+              __builtin_amdgcn_sched_barrier(0);
+              o[i * NRBW + j] = mfma16<F16>(va_cur, pbv[j], o[i * NRBW + j]);
+              if (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
+#if !defined(DG_EXP) || DG_EXP != 3
+              if (n % LDV_EVERY == 0 && n / LDV_EVERY < NLD) issue_tile_part<D, true>(next_v, n / LDV_EVERY, wave, lane_l);
+#endif
+            }
+            va_cur = va_next;
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
 #ifdef DG_ATTN_PHASE_TIMING
-      asm volatile("s_nop 0" ::"a"(o[0][0]), "a"(o[NDB - 1][15]));
+      asm volatile("s_nop 0" ::"a"(o[0][0]), "a"(o[NACC - 1][15]));
 #endif
       DG_PHASE(6)
       if constexpr (PIPE) {
@@ -458,52 +526,70 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 
   // ---- epilogue ----
   DG_PHASE_STORE
+  // row owners publish (m, l) of their rows; d owners normalise and store their slice of O
   const float l_tot = sum_across_halves(l_part);
-  if (p.n_splits > 1) {
-    const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + r;
-    float* po = p.part_o + prow * D + 4u * g2;
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        f32x4 v4 = {o[db][4 * q4], o[db][4 * q4 + 1], o[db][4 * q4 + 2], o[db][4 * q4 + 3]};
-        *(f32x4*)(po + 32 * db + 8 * q4) = v4;
-      }
-    if (g2 == 0) {
+  __syncthreads();   // the last tile's readers are done with LDS
+  if (g2 == 0) {
+    sml[(wave * 32u + l32) * 2u] = m_ref;
+    sml[(wave * 32u + l32) * 2u + 1u] = l_tot;
+    if (p.n_splits > 1) {
+      const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + r;
       p.part_ml[prow * 2] = m_ref;
       p.part_ml[prow * 2 + 1] = l_tot;
+    } else if (row_ok) {
+      if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l_tot > 0.f ? m_ref * kLn2 + __logf(l_tot) : -INFINITY;
+      if (p.dbg && !(l_tot > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l_tot));
     }
-    return;
   }
-  if (!row_ok) return;
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  const size_t ooff = ((size_t)tok * p.hq + qh) * D + 4u * g2;
-  if (g2 == 0) {
-    if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l_tot > 0.f ? m_ref * kLn2 + __logf(l_tot) : -INFINITY;
-    if (p.dbg && !(l_tot > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l_tot));
-  }
+  __syncthreads();
 #pragma unroll
-  for (int db = 0; db < NDB; ++db)
+  for (int j = 0; j < NRBW; ++j) {
+    const uint32_t rbk = rgrp * NRBW + j;
+    const uint32_t rr = row0 + rbk * 32u + l32;
+    if (p.n_splits > 1) {
+      const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + rr;
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const float y0 = o[db][4 * q4] * inv, y1 = o[db][4 * q4 + 1] * inv;
-      const float y2 = o[db][4 * q4 + 2] * inv, y3 = o[db][4 * q4 + 3] * inv;
-      const size_t idx = ooff + 32 * db + 8 * q4;
-      if (p.out_dtype == DT_F32) {
-        f32x4 v4 = {y0, y1, y2, y3};
-        *(f32x4*)((float*)p.out + idx) = v4;
-      } else {
-        u32x2 pk;
-        if (p.out_trunc) {
-          pk[0] = (__float_as_uint(y0) >> 16) | (__float_as_uint(y1) & 0xffff0000u);
-          pk[1] = (__float_as_uint(y2) >> 16) | (__float_as_uint(y3) & 0xffff0000u);
-        } else {
-          pk[0] = pack2<false>(y0, y1);
-          pk[1] = pack2<false>(y2, y3);
+      for (int i = 0; i < NDBW; ++i) {
+        float* po = p.part_o + prow * D + 32u * (dgrp * NDBW + i) + 4u * g2;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x16& a = o[i * NRBW + j];
+          f32x4 v4 = {a[4 * q4], a[4 * q4 + 1], a[4 * q4 + 2], a[4 * q4 + 3]};
+          *(f32x4*)(po + 8 * q4) = v4;
         }
-        *(u32x2*)((uint16_t*)p.out + idx) = pk;
+      }
+      continue;
+    }
+    if (rr >= p.rows_total) continue;
+    const float l_row = sml[(rbk * 32u + l32) * 2u + 1u];
+    const float inv = l_row > 0.f ? 1.f / l_row : 0.f;
+    const uint32_t tok_o = rr / p.group, qh_o = kvh * p.group + rr % p.group;
+#pragma unroll
+    for (int i = 0; i < NDBW; ++i) {
+      const size_t idx0 = ((size_t)tok_o * p.hq + qh_o) * D + 32u * (dgrp * NDBW + i) + 4u * g2;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const f32x16& a = o[i * NRBW + j];
+        const float y0 = a[4 * q4] * inv, y1 = a[4 * q4 + 1] * inv;
+        const float y2 = a[4 * q4 + 2] * inv, y3 = a[4 * q4 + 3] * inv;
+        const size_t idx = idx0 + 8 * q4;
+        if (p.out_dtype == DT_F32) {
+          f32x4 v4 = {y0, y1, y2, y3};
+          *(f32x4*)((float*)p.out + idx) = v4;
+        } else {
+          u32x2 pk;
+          if (p.out_trunc) {
+            pk[0] = (__float_as_uint(y0) >> 16) | (__float_as_uint(y1) & 0xffff0000u);
+            pk[1] = (__float_as_uint(y2) >> 16) | (__float_as_uint(y3) & 0xffff0000u);
+          } else {
+            pk[0] = pack2<false>(y0, y1);
+            pk[1] = pack2<false>(y2, y3);
+          }
+          *(u32x2*)((uint16_t*)p.out + idx) = pk;
+        }
       }
     }
+  }
 }
 
 template <int D, bool F16>
