@@ -33,6 +33,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline sample time")
     ap.add_argument("--check-toks", type=int, default=12)
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="instead of the benchmark, run the library's plain copy kernel over this many MiB "
+                         "(the known-size launch the profiler's HBM byte counters are scaled by)")
     return ap.parse_args()
 
 
@@ -71,6 +74,18 @@ def main():
         sys.exit(3)
     from diffgemma_amd import attention as A, capi, workloads as W
     from oracle import pyoracle as po
+
+    if args.calib_copy_mib > 0:
+        nbytes = args.calib_copy_mib << 20
+        src = torch.ones(nbytes, dtype=torch.uint8, device="cuda")
+        dst = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        for _ in range(args.steps):
+            capi.check(capi.load().dg_calib_copy(dst.data_ptr(), src.data_ptr(), nbytes, A.stream_handle()))
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        print(json.dumps({"calib_copy_bytes": nbytes, "launches": args.steps, "kernel": "calib_copy_kernel"}))
+        return
 
     w = W.config(args.workload)
     t_gen = time.perf_counter()

@@ -19,8 +19,13 @@
 //
 // K and V tiles arrive by 16-byte direct-to-LDS loads, double buffered, issued one instruction
 // at a time between MFMAs.  The running max is only raised (and O rescaled) when some row's
-// tile max exceeds it by more than 2^kTau, which in steady state is never; the raise is
-// broadcast to the d owners through LDS together with P.
+// tile max exceeds it by more than 2^tau; the raise is broadcast to the d owners through LDS
+// together with P.  Rescaling O costs about as much as the tile's P.V MFMAs, and with unit-RMS
+// Q and K and no 1/sqrt(d) the scores of a row spread over tens of log2 units, so a small tau
+// would rescale some row block on almost every tile.  Any reference below the true max is
+// exact as long as nothing overflows: P <= 2^tau, and the fp32 sums stay below
+// 2^tau * keys * |v|, far from 2^127 for tau = 64.  With f16 operands P itself has to stay
+// below 65504.
 #include "attn_params.h"
 
 namespace dg {
@@ -40,7 +45,9 @@ typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 typedef __attribute__((address_space(1))) const void gbl_void;
 typedef __attribute__((address_space(3))) void lds_void;
 
-constexpr float kTau = 8.0f;  // log2 units: P never exceeds 2^8 before a rescale
+// log2 units by which a tile max may exceed the reference max before the reference is raised
+template <bool F16>
+constexpr float kTau = F16 ? 12.0f : 64.0f;
 
 // Optional per-phase cycle accounting (development builds only): every wave sums the cycles
 // it spends in each phase of the tile loop and stores the sums at the end.
@@ -100,6 +107,26 @@ __device__ __forceinline__ float unpack_hi(uint32_t u) {
 // s_waitcnt vmcnt(0) as a builtin, so that the compiler's own wait-count bookkeeping sees it
 // (gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt = 6:4, lgkmcnt = 11:8; the other two
 // counters are left at their maxima).
+// acc + lo + hi of a packed pair, in one dot-product instruction
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <bool F16>
+__device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
+  if constexpr (F16) {
+    const f16x2_t ones = {(_Float16)1.f, (_Float16)1.f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, pk), ones, acc, false);
+  } else {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u),
+                                           acc, false);
+  }
+}
+
+// wait until at most N of this wave's vector memory loads are outstanding (N <= 15)
+template <int N>
+__device__ __forceinline__ void wait_vmem_but() {
+  static_assert(N >= 0 && N <= 15, "vmcnt immediate");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+}
 __device__ __forceinline__ void wait_vmem_all() {
   __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("" ::: "memory");
@@ -117,39 +144,56 @@ __device__ __forceinline__ float sum_across_halves(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// 16-byte chunk swizzles of a tile row (CPR = chunks per row).  K is read as 32 rows x one
-// chunk per half-wave, V as 8 rows x 4 chunks per transpose read; both patterns then fall
-// on distinct banks.
-template <int CPR>
-__device__ __forceinline__ uint32_t swz_k(uint32_t row) {
-  if constexpr (CPR >= 16) return row & 15u;
-  else return (row / (16 / CPR)) & (CPR - 1);
-}
-template <int CPR>
-__device__ __forceinline__ uint32_t swz_v(uint32_t row) {
-  return ((row & 3u) << 2) & (CPR - 1);
-}
+// LDS layout of one 32-key tile of K or V (rows = keys, head_dim contiguous, 16-byte chunks).
+//
+// head_dim 512: a row is exactly the KiB one direct-to-LDS instruction writes, so rows can be
+// padded apart: K rows by 16 B (32 rows x one chunk per half-wave fall on distinct banks),
+// V rows by 64 B (the 8 rows x 4 chunks of a transposing read do).  Every fragment address is
+// then one per-lane base plus a compile-time offset, and the global side of a load is one
+// row: a scalar address plus lane*16.
+// smaller head_dim: several rows share an instruction's KiB, so rows stay dense and the 16-byte
+// chunks are XOR-swizzled instead (the swizzle is applied by choosing which global chunk each
+// lane fetches).
+template <int D>
+struct Lay {
+  static constexpr int CPR = D / 8;          // chunks per row
+  static constexpr int ROWB = 2 * D;         // bytes per row
+  static constexpr bool PAD = CPR == 64;
+  static constexpr int K_STRIDE = PAD ? ROWB + 16 : ROWB;
+  static constexpr int V_STRIDE = PAD ? ROWB + 64 : ROWB;
+  static constexpr int K_BYTES = 32 * K_STRIDE, V_BYTES = 32 * V_STRIDE;
+  static constexpr int NBLK = 32 * CPR / 64;   // KiB blocks (= load instructions) per tile
+  static constexpr int NLD = (NBLK + 3) / 4;   // load instructions per wave and tile
+  static __device__ __forceinline__ uint32_t swz_k(uint32_t row) {
+    if constexpr (PAD) return 0u;
+    else if constexpr (CPR >= 16) return row & 15u;
+    else return (row / (16 / CPR)) & (CPR - 1);
+  }
+  static __device__ __forceinline__ uint32_t swz_v(uint32_t row) {
+    if constexpr (PAD) return 0u;
+    else return ((row & 3u) << 2) & (CPR - 1);
+  }
+};
 
-// One 32-key tile's direct-to-LDS loads, described once per tile and issued one wave
-// instruction at a time so the issue slots can be spread between MFMAs.  Each instruction
-// fills one contiguous KiB of LDS (64 lanes x 16 B); the swizzle is applied by choosing which
-// global chunk each lane fetches.  Keys past t_all re-read key t_all-1 (finite, masked later).
+// One tile's direct-to-LDS loads, described once per tile and issued one wave instruction at a
+// time so the issue slots can be spread between MFMAs.  Keys past t_all re-read key t_all-1
+// (finite data, masked later).
 struct TileLoad {
   const char* base;   // head base + slot(t0) * row stride (wave-uniform)
-  uint32_t stride_b;  // bytes between key rows
+  uint32_t stride_b;  // bytes between key rows in global memory
   uint32_t rmax;      // last valid row of the tile
   uint32_t lds;       // LDS byte address of the destination buffer
-  bool on;
+  uint32_t rot;       // rotation of the order in which the tile's KiB blocks are fetched
 };
 
 __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_t tok_stride_b, uint32_t t0,
-                                                   uint32_t t_all, uint32_t ring_mask, lds_char* buf, bool on) {
+                                                   uint32_t t_all, uint32_t ring_mask, lds_char* buf, uint32_t rot) {
   TileLoad tl;
   tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
   tl.stride_b = (uint32_t)tok_stride_b;
   tl.rmax = t_all - 1u - t0;
   tl.lds = (uint32_t)(size_t)buf;
-  tl.on = on;
+  tl.rot = rot;
   return tl;
 }
 
@@ -157,25 +201,12 @@ __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_
 // direct-to-LDS load it knows about with s_waitcnt vmcnt(0), which would expose the whole
 // fetch latency once per tile.  The kernel waits for these loads itself, at the top of the
 // tile loop, one iteration after they were issued.
-template <int D, bool IS_V>
-__device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint32_t wave, uint32_t lane) {
-  constexpr int CPR = D / 8;
-  constexpr int NBLK = 32 * CPR / 64;
-  if (!tl.on) return;
-#if defined(DG_EXP) && DG_EXP == 1
-  return;   // experiment: no tile loads inside the loop
-#endif
-  const uint32_t blk = k * 4 + wave;
-  if (NBLK < 4 && blk >= (uint32_t)NBLK) return;
-  const uint32_t pch = blk * 64 + lane;
-  const uint32_t r = pch / CPR, pc = pch % CPR;
-  const uint32_t c = pc ^ (IS_V ? swz_v<CPR>(r) : swz_k<CPR>(r));
-  const uint32_t voff = min(r, tl.rmax) * tl.stride_b + c * 16u;
-  // both are wave-uniform by construction; readfirstlane tells the compiler so
-  const uint32_t dst = __builtin_amdgcn_readfirstlane(tl.lds + blk * 1024u);
-  const uint64_t b = (uint64_t)tl.base;
-  // (readfirstlane returns a signed int: without the casts the low half would be sign-extended
-  // over the high half)
+__device__ __forceinline__ void lds_dma_16(const char* base_uniform, uint32_t voff, uint32_t lds_dst_uniform) {
+  // all scalar operands are wave-uniform by construction; readfirstlane tells the compiler so
+  // (it returns a signed int: without the casts the low half would be sign-extended over the
+  // high half)
+  const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_dst_uniform);
+  const uint64_t b = (uint64_t)base_uniform;
   const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32) |
                         (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base)
@@ -183,30 +214,52 @@ __device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint3
 }
 
 template <int D, bool IS_V>
+__device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint32_t wave, uint32_t lane) {
+  using L = Lay<D>;
+  if (L::NBLK < 4 && k * 4 + wave >= (uint32_t)L::NBLK) return;
+  // Workgroups that stream the same keys run in near lockstep; each starts its tile at a
+  // different block so that they do not all ask the L2 for the same lines at the same time.
+  const uint32_t blk = (k * 4 + wave + tl.rot) & (uint32_t)(L::NBLK - 1);
+  if constexpr (L::PAD) {
+    // one instruction = one key row: the row part of the address is scalar
+    const char* row = tl.base + (uint64_t)min(blk, tl.rmax) * tl.stride_b;
+    lds_dma_16(row, lane * 16u, tl.lds + blk * (IS_V ? L::V_STRIDE : L::K_STRIDE));
+  } else {
+    const uint32_t pch = blk * 64 + lane;
+    const uint32_t r = pch / L::CPR, pc = pch % L::CPR;
+    const uint32_t c = pc ^ (IS_V ? L::swz_v(r) : L::swz_k(r));
+    lds_dma_16(tl.base, min(r, tl.rmax) * tl.stride_b + c * 16u, tl.lds + blk * 1024u);
+  }
+}
+
+template <int D, bool IS_V>
 __device__ __forceinline__ void issue_tile(const TileLoad& tl, uint32_t wave, uint32_t lane) {
-  constexpr int NLD = (32 * (D / 8) / 64 + 3) / 4;
 #pragma unroll
-  for (int k = 0; k < NLD; ++k) issue_tile_part<D, IS_V>(tl, k, wave, lane);
+  for (int k = 0; k < Lay<D>::NLD; ++k) issue_tile_part<D, IS_V>(tl, k, wave, lane);
 }
 
 // PIPE: issue Q.K^T of tile j+1 before the softmax of tile j (needs a second score tile in
 // registers; used where the register file has room for it).
 template <int D, bool F16, bool PIPE>
 __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
-  constexpr int CPR = D / 8, ROWB = 2 * D, TILEB = kBlockN * ROWB, NSTEP = D / 16, NDB = D / 32;
+  using L = Lay<D>;
+  constexpr int NSTEP = D / 16, NDB = D / 32;
   // P.V work split: DSPLIT groups of d-blocks x RSPLIT groups of row-blocks = 4 waves
   constexpr int DSPLIT = NDB < 4 ? NDB : 4, RSPLIT = 4 / DSPLIT;
   constexpr int NDBW = NDB / DSPLIT;   // d-blocks (32 wide) this wave accumulates
   constexpr int NRBW = 4 / RSPLIT;     // row-blocks (32 rows) this wave accumulates
   constexpr int NACC = NDBW * NRBW;
-  __shared__ __attribute__((aligned(1024))) char sk0[TILEB];
-  __shared__ __attribute__((aligned(1024))) char sk1[TILEB];
-  __shared__ __attribute__((aligned(1024))) char sv0[TILEB];
-  __shared__ __attribute__((aligned(1024))) char sv1[TILEB];
-  __shared__ __attribute__((aligned(1024))) char sp[2 * 4 * 1024];   // P: [ks][row-block][lane] x 16 B
-  __shared__ __attribute__((aligned(16))) float scorr[4 * 32];       // per-row rescale factor of this tile
-  __shared__ __attribute__((aligned(16))) uint32_t sflag[4];         // row-block raised its max this tile
-  __shared__ __attribute__((aligned(16))) float sml[4 * 32 * 2];     // epilogue: (m, l) per row
+  // One LDS block, carved by hand so that the order of the buffers is fixed:
+  //   K0 K1 | V0 V1 | P: [ks][row-block][lane] x 16 B | per-row rescale factor of this tile |
+  //   "row-block raised its max this tile" flags | epilogue (m, l) per row
+  constexpr int OFF_K0 = 0, OFF_K1 = L::K_BYTES, OFF_V0 = 2 * L::K_BYTES, OFF_V1 = OFF_V0 + L::V_BYTES;
+  constexpr int OFF_P = 2 * L::K_BYTES + 2 * L::V_BYTES, OFF_CORR = OFF_P + 2 * 4 * 1024;
+  constexpr int OFF_FLAG = OFF_CORR + 4 * 32 * 4, OFF_ML = OFF_FLAG + 16, LDS_BYTES = OFF_ML + 4 * 32 * 2 * 4;
+  static_assert(L::K_BYTES % 16 == 0 && L::V_BYTES % 16 == 0, "buffer alignment");
+  __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
+  float* const scorr = (float*)(smem + OFF_CORR);
+  uint32_t* const sflag = (uint32_t*)(smem + OFF_FLAG);
+  float* const sml = (float*)(smem + OFF_ML);
 
   // ---- which (KV head, split, row tile) this workgroup owns ----
   // Workgroup ids go round-robin over the 8 XCDs.  All row tiles of one (KV head, split)
@@ -297,32 +350,43 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const char* vbase = (const char*)p.v + (int64_t)kvh * p.v_head_stride * 2;
   const int64_t kstride_b = p.k_tok_stride * 2, vstride_b = p.v_tok_stride * 2;
 
-  // per-lane LDS byte offsets of the fragment reads
-  const uint32_t k_row_off = l32 * ROWB;
-  const uint32_t k_swz = swz_k<CPR>(l32);
+  // per-lane LDS byte offsets of the fragment reads (everything else is a compile-time offset
+  // in the padded layout, or one XOR with a per-lane constant in the swizzled one)
+  const uint32_t k_lane_off = l32 * L::K_STRIDE + (L::PAD ? g2 * 16u : 0u);
+  const uint32_t k_swz = L::swz_k(l32);
   const uint32_t v_row = 4u * g2 + (i16 >> 2);  // + 16*ks + 8*q, which keeps row&3
-  const uint32_t v_swz = swz_v<CPR>(v_row);
+  const uint32_t v_swz = L::swz_v(v_row);
   const uint32_t v_lane_chunk = 2u * h16 + ((i16 & 3u) >> 1);
-  const uint32_t v_lane_off = v_row * ROWB + (i16 & 1u) * 8u;
-  lds_char* const pbuf = (lds_char*)sp;
+  const uint32_t v_lane_off = v_row * L::V_STRIDE + (i16 & 1u) * 8u + (L::PAD ? v_lane_chunk * 16u : 0u);
+  lds_char* const pbuf = (lds_char*)(smem + OFF_P);
 
-  constexpr int NLD = (32 * CPR / 64 + 3) / 4;   // load instructions per wave, tile and matrix
+  constexpr int NLD = L::NLD;                    // load instructions per wave, tile and matrix
   constexpr int NQK = NSTEP, NPV = 2 * NACC;     // MFMAs per wave and tile in each phase
-  constexpr int PFK = NQK < 4 ? NQK : 4;         // K fragment reads kept in flight ahead of the MFMAs
+  constexpr int PFK = NQK < 8 ? NQK : 8;         // K fragment reads kept in flight ahead of the MFMAs
   constexpr int LDK_EVERY = NQK / NLD, LDV_EVERY = NPV / NLD;
 
+  // K fragment of MFMA step st: A operand, lane = key row l32, 8 consecutive d at 16*st + 8*g2
   auto k_frag = [&](lds_char* kb, int st) -> u32x4 {
-    const uint32_t c = (uint32_t)(2 * st) + g2;
-    return *(lds_u32x4*)(kb + k_row_off + ((c ^ k_swz) << 4));
+    if constexpr (L::PAD) {
+      return *(lds_u32x4*)(kb + k_lane_off + 32 * st);
+    } else {
+      const uint32_t c = (uint32_t)(2 * st) + g2;
+      return *(lds_u32x4*)(kb + k_lane_off + ((c ^ k_swz) << 4));
+    }
   };
   // V^T fragment for MFMA k-step ks of d-block db: k-slot j of lane half g2 is key
   // 16*ks + 8*(j>>2) + 4*g2 + (j&3), the order in which the score accumulator holds keys.
   auto v_frag = [&](lds_char* vb, int ks, uint32_t db) -> u32x4 {
-    const uint32_t c = 4u * db + v_lane_chunk;
-    const uint32_t off = v_lane_off + (uint32_t)(16 * ks) * ROWB + ((c ^ v_swz) << 4);
+    uint32_t off;
+    if constexpr (L::PAD) {
+      off = v_lane_off + (uint32_t)(16 * ks) * L::V_STRIDE + 64u * db;
+    } else {
+      const uint32_t c = 4u * db + v_lane_chunk;
+      off = v_lane_off + (uint32_t)(16 * ks) * L::V_STRIDE + ((c ^ v_swz) << 4);
+    }
     const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off)));
-    const u32x2 hi =
-        __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off + 8 * ROWB)));
+    const u32x2 hi = __builtin_bit_cast(
+        u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off + 8 * L::V_STRIDE)));
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
   auto p_frag = [&](int ks, uint32_t rbk) -> u32x4 {
@@ -332,7 +396,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   // S^T = K.Q^T for one tile.  PFK fragment reads run ahead of the MFMA that consumes them and
   // the next K tile's global loads are issued one instruction every LDK_EVERY MFMAs; the
   // scheduling barriers keep that interleaving.
-  auto qk_tile = [&](lds_char* kb, const TileLoad& next_k, uint32_t ld_lane) -> f32x16 {
+  auto qk_tile = [&](lds_char* kb, const TileLoad& next_k, uint32_t ld_lane, bool with_loads) -> f32x16 {
     f32x16 s;
 #pragma unroll
     for (int e = 0; e < 16; ++e) s[e] = 0.f;
@@ -344,9 +408,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       __builtin_amdgcn_sched_barrier(0);
       s = mfma16<F16>(kf[st % PFK], qf[st], s);
       if (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
-#if !defined(DG_EXP) || DG_EXP != 3
-      if (st % LDK_EVERY == 0 && st / LDK_EVERY < NLD) issue_tile_part<D, false>(next_k, st / LDK_EVERY, wave, ld_lane);
-#endif
+      if (with_loads && st % LDK_EVERY == 0 && st / LDK_EVERY < NLD)
+        issue_tile_part<D, false>(next_k, st / LDK_EVERY, wave, ld_lane);
     }
     __builtin_amdgcn_sched_barrier(0);
     return s;
@@ -354,59 +417,61 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 
   DG_PHASE_DECL
   if (ntile > 0) {
-    lds_char* const k0 = (lds_char*)sk0;
-    lds_char* const k1 = (lds_char*)sk1;
-    lds_char* const v0 = (lds_char*)sv0;
-    lds_char* const v1 = (lds_char*)sv1;
-    const TileLoad none = make_tile_load(kbase, kstride_b, tb * kBlockN, p.t_all, p.ring_mask, k0, false);
+    lds_char* const k0 = (lds_char*)(smem + OFF_K0);
+    lds_char* const k1 = (lds_char*)(smem + OFF_K1);
+    lds_char* const v0 = (lds_char*)(smem + OFF_V0);
+    lds_char* const v1 = (lds_char*)(smem + OFF_V1);
+    // Loads for a tile past the last one are not branched around: they fetch the last tile
+    // again into a buffer nobody reads any more.
+    const uint32_t t_last = (te - 1u) * kBlockN;
+    const uint32_t ld_rot = (mt * (L::NBLK >= 32 ? 2u : 1u)) & (uint32_t)(L::NBLK - 1);
+    auto k_load = [&](uint32_t t0, lds_char* buf) {
+      return make_tile_load(kbase, kstride_b, min(t0, t_last), p.t_all, p.ring_mask, buf, ld_rot);
+    };
+    auto v_load = [&](uint32_t t0, lds_char* buf) {
+      return make_tile_load(vbase, vstride_b, min(t0, t_last), p.t_all, p.ring_mask, buf, ld_rot);
+    };
 
-    issue_tile<D, false>(make_tile_load(kbase, kstride_b, tb * kBlockN, p.t_all, p.ring_mask, k0, true), wave, lane);
-    if (ntile > 1)
-      issue_tile<D, false>(make_tile_load(kbase, kstride_b, (tb + 1) * kBlockN, p.t_all, p.ring_mask, k1, true), wave, lane);
-    issue_tile<D, true>(make_tile_load(vbase, vstride_b, tb * kBlockN, p.t_all, p.ring_mask, v0, true), wave, lane);
+    issue_tile<D, false>(k_load(tb * kBlockN, k0), wave, lane);
+    if constexpr (PIPE) issue_tile<D, false>(k_load((tb + 1) * kBlockN, k1), wave, lane);
+    issue_tile<D, true>(v_load(tb * kBlockN, v0), wave, lane);
     wait_vmem_all();
     __syncthreads();
     f32x16 s_cur;
     if constexpr (PIPE) {
       // K(tb+2) goes where K(tb) sits, so it cannot be issued before this first tile is consumed
-      s_cur = qk_tile(k0, none, lane);
+      s_cur = qk_tile(k0, k_load(0, k0), lane, false);
     }
     DG_PHASE(0)
 
     for (uint32_t jj = 0; jj < ntile; ++jj) {
       const uint32_t t0 = (tb + jj) * kBlockN;
       lds_char* const kb_even = (jj & 1u) ? k1 : k0;   // holds K(jj)
-      lds_char* const kb_odd = (jj & 1u) ? k0 : k1;    // holds K(jj+1)
+      lds_char* const kb_odd = (jj & 1u) ? k0 : k1;    // holds K(jj+1) (PIPE) or takes it
       lds_char* const vb_cur = (jj & 1u) ? v1 : v0;    // holds V(jj)
       lds_char* const vb_free = (jj & 1u) ? v0 : v1;   // refill with V(jj+1)
 
-      // Barrier A: the tiles this iteration reads have landed everywhere, and every wave is done
-      // with the previous tile (its K/V buffers, the P tile and the rescale words can be reused).
-      wait_vmem_all();
+      // Barrier A: the K tile this iteration multiplies has landed everywhere (this wave's share
+      // of it is older than its NLD loads of V(jj), which may still be in flight), and every wave
+      // is done with the previous tile (its K/V buffers, the P tile and the rescale words can be
+      // reused).
+      wait_vmem_but<NLD>();
       DG_PHASE(1)
       __syncthreads();
       DG_PHASE(2)
       // Re-derive the per-lane global offsets of the tile loads inside every iteration: hoisted
-      // out of the loop they would cost sixteen more live VGPRs than this kernel has.
+      // out of the loop they would cost more live VGPRs than this kernel has.
       uint32_t lane_l = lane;
       asm volatile("" : "+v"(lane_l));
       // PIPE: K(jj) was consumed one iteration ago, its buffer takes K(jj+2).
-      // otherwise: K(jj+1) goes to the other buffer (the prologue already fetched K(tb+1)).
-      const TileLoad next_k =
-          PIPE ? make_tile_load(kbase, kstride_b, t0 + 2 * kBlockN, p.t_all, p.ring_mask, kb_even, jj + 2 < ntile)
-               : make_tile_load(kbase, kstride_b, t0 + kBlockN, p.t_all, p.ring_mask, kb_odd,
-                                jj >= 1 && jj + 1 < ntile);
-      const TileLoad next_v =
-          make_tile_load(vbase, vstride_b, t0 + kBlockN, p.t_all, p.ring_mask, vb_free, jj + 1 < ntile);
-#if defined(DG_EXP) && DG_EXP == 3
-      issue_tile<D, false>(next_k, wave, lane_l);
-      issue_tile<D, true>(next_v, wave, lane_l);
-#endif
+      // otherwise: K(jj+1) goes to the other buffer while K(jj) is read.
+      const TileLoad next_k = PIPE ? k_load(t0 + 2 * kBlockN, kb_even) : k_load(t0 + kBlockN, kb_odd);
+      const TileLoad next_v = v_load(t0 + kBlockN, vb_free);
       f32x16 s_next;
       if constexpr (PIPE) {
-        if (jj + 1 < ntile) s_next = qk_tile(kb_odd, next_k, lane_l);
+        if (jj + 1 < ntile) s_next = qk_tile(kb_odd, next_k, lane_l, true);
       } else {
-        s_cur = qk_tile(kb_even, next_k, lane_l);
+        s_cur = qk_tile(kb_even, next_k, lane_l, true);
       }
 #ifdef DG_ATTN_PHASE_TIMING
       asm volatile("s_nop 0" ::"v"(s_cur[0]), "v"(s_cur[15]));  // the scores have to exist before the clock is read
@@ -427,7 +492,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
       for (int e = 1; e < 16; ++e) tmax = fmaxf(tmax, s_cur[e]);
       tmax = max_across_halves(tmax) * p.scale_log2;
-      const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau) != 0ull;
+      const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau<F16>) != 0ull;
       if (raise) {
         const float m_new = fmaxf(m_ref, tmax);
         const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -448,13 +513,16 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           const uint32_t pk = pack2<F16>(p0, p1);
           pk4[j >> 1] = pk;
           // the row sum uses the rounded probabilities, the same numbers P.V multiplies
-          l_part += unpack_lo<F16>(pk) + unpack_hi<F16>(pk);
+          l_part = add_pair<F16>(pk, l_part);
         }
         // register image of the B operand of MFMA k-step ks for (row l32, lane half g2)
         *(lds_u32x4*)(pbuf + (((uint32_t)ks * 4u + wave) * 64u + lane) * 16u) = pk4;
       }
       DG_PHASE(4)
-      // Barrier B: P and the rescale words of this tile are visible to the d owners.
+      // Barrier B: P and the rescale words of this tile are visible to the d owners, and V(jj)
+      // has landed everywhere (only the NLD loads of the next K tile, issued after it, may still
+      // be in flight).
+      wait_vmem_but<NLD>();
       __syncthreads();
       DG_PHASE(5)
 
@@ -485,32 +553,31 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           }
         }
         // O^T += V^T . P^T: per k-step, NDBW V^T fragments x NRBW P fragments.  The P fragments
-        // of a k-step stay in registers for the whole step; the V^T fragment of the next d-block
-        // is fetched while the current one multiplies, and each P fragment of k-step 1 replaces
-        // its k-step 0 counterpart right after that one's last use.  V(jj+1)'s global loads are
-        // spread between the MFMAs.
+        // of a k-step stay in registers for the whole step; V^T fragments are fetched PFV ahead
+        // of the one that multiplies, and each P fragment of k-step 1 replaces its k-step 0
+        // counterpart right after that one's last use.  V(jj+1)'s global loads are spread between
+        // the MFMAs.
+        constexpr int NVF = 2 * NDBW;                    // V^T fragments per tile and wave
+        constexpr int PFV = NVF - 1 < 3 ? NVF - 1 : 3;   // fragment reads in flight ahead of the MFMAs
+        auto v_frag_n = [&](int f) { return v_frag(vb_cur, f / NDBW, dgrp * NDBW + f % NDBW); };
         u32x4 pbv[NRBW];
 #pragma unroll
         for (int j = 0; j < NRBW; ++j) pbv[j] = p_frag(0, rgrp * NRBW + j);
-        u32x4 va_cur = v_frag(vb_cur, 0, dgrp * NDBW), va_next = va_cur;
+        u32x4 va[PFV + 1];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int f = 0; f <= PFV; ++f) va[f] = v_frag_n(f);
 #pragma unroll
-          for (int i = 0; i < NDBW; ++i) {
-            const int nxt = ks * NDBW + i + 1;   // next (k-step, d-block) pair
-            if (nxt < 2 * NDBW) va_next = v_frag(vb_cur, nxt / NDBW, dgrp * NDBW + nxt % NDBW);
+        for (int f = 0; f < NVF; ++f) {
+          const int ks = f / NDBW, i = f % NDBW;
 #pragma unroll
-            for (int j = 0; j < NRBW; ++j) {
-              const int n = (ks * NDBW + i) * NRBW + j;   // MFMA index within the tile
-              __builtin_amdgcn_sched_barrier(0);
-              o[i * NRBW + j] = mfma16<F16>(va_cur, pbv[j], o[i * NRBW + j]);
-              if (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
-#if !defined(DG_EXP) || DG_EXP != 3
-              if (n % LDV_EVERY == 0 && n / LDV_EVERY < NLD) issue_tile_part<D, true>(next_v, n / LDV_EVERY, wave, lane_l);
-#endif
-            }
-            va_cur = va_next;
+          for (int j = 0; j < NRBW; ++j) {
+            const int n = f * NRBW + j;   // MFMA index within the tile
+            __builtin_amdgcn_sched_barrier(0);
+            o[i * NRBW + j] = mfma16<F16>(va[f % (PFV + 1)], pbv[j], o[i * NRBW + j]);
+            if (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
+            if (n % LDV_EVERY == 0 && n / LDV_EVERY < NLD) issue_tile_part<D, true>(next_v, n / LDV_EVERY, wave, lane_l);
           }
+          if (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -522,6 +589,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         if (jj + 1 < ntile) s_cur = s_next;
       }
     }
+    // the loads issued for the tile after the last one must not outlive this workgroup's LDS
+    wait_vmem_all();
   }
 
   // ---- epilogue ----

@@ -430,6 +430,12 @@ int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches) {
   return rc;
 }
 
+int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream) {
+  if (!dst || !src) return DG_ERR_NULL;
+  if (bytes % 16 != 0 || ((uintptr_t)dst % 16) != 0 || ((uintptr_t)src % 16) != 0) return DG_ERR_LAYOUT;
+  return dg::launch_calib_copy(dst, src, bytes, (hipStream_t)stream) == hipSuccess ? DG_OK : DG_ERR_LAUNCH;
+}
+
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype) { return (uint64_t)head_dim * elem_size(kv_dtype); }
 
 uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slots, uint32_t kv_dtype) {

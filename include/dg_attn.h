@@ -168,6 +168,11 @@ int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims
 int dg_prof_begin(uint32_t max_launches);
 int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches);
 
+/* Plain device-to-device copy of `bytes` (multiple of 16) with a kernel of this library: a
+ * launch of known HBM traffic (bytes read + bytes written) that the FETCH_SIZE / WRITE_SIZE
+ * profiler counters are scaled by.  Measurement aid, no counterpart in the reference. */
+int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);
 uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slots, uint32_t kv_dtype);
