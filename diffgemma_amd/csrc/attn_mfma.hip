@@ -176,21 +176,26 @@ struct Lay {
 };
 
 // One tile's direct-to-LDS loads, described once per tile and issued one wave instruction at a
-// time so the issue slots can be spread between MFMAs.  Keys past t_all re-read key t_all-1
-// (finite data, masked later).
+// time so the issue slots can be spread between MFMAs.  Rows of the tile outside
+// [t_min, t_all) are replaced by the nearest row inside: those keys are masked for every query
+// row of the workgroup, but what their slots hold (dead ring slots, memory past the cache) may
+// not be finite, and 0 * NaN would poison P.V.
 struct TileLoad {
   const char* base;   // head base + slot(t0) * row stride (wave-uniform)
   uint32_t stride_b;  // bytes between key rows in global memory
-  uint32_t rmax;      // last valid row of the tile
+  uint32_t rmin;      // first row of the tile that may be read
+  uint32_t rmax;      // last row of the tile that may be read
   uint32_t lds;       // LDS byte address of the destination buffer
   uint32_t rot;       // rotation of the order in which the tile's KiB blocks are fetched
 };
 
 __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_t tok_stride_b, uint32_t t0,
-                                                   uint32_t t_all, uint32_t ring_mask, lds_char* buf, uint32_t rot) {
+                                                   uint32_t t_min, uint32_t t_all, uint32_t ring_mask, lds_char* buf,
+                                                   uint32_t rot) {
   TileLoad tl;
   tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
   tl.stride_b = (uint32_t)tok_stride_b;
+  tl.rmin = t_min > t0 ? t_min - t0 : 0u;
   tl.rmax = t_all - 1u - t0;
   tl.lds = (uint32_t)(size_t)buf;
   tl.rot = rot;
@@ -222,13 +227,13 @@ __device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint3
   const uint32_t blk = (k * 4 + wave + tl.rot) & (uint32_t)(L::NBLK - 1);
   if constexpr (L::PAD) {
     // one instruction = one key row: the row part of the address is scalar
-    const char* row = tl.base + (uint64_t)min(blk, tl.rmax) * tl.stride_b;
+    const char* row = tl.base + (uint64_t)min(max(blk, tl.rmin), tl.rmax) * tl.stride_b;
     lds_dma_16(row, lane * 16u, tl.lds + blk * (IS_V ? L::V_STRIDE : L::K_STRIDE));
   } else {
     const uint32_t pch = blk * 64 + lane;
     const uint32_t r = pch / L::CPR, pc = pch % L::CPR;
     const uint32_t c = pc ^ (IS_V ? L::swz_v(r) : L::swz_k(r));
-    lds_dma_16(tl.base, min(r, tl.rmax) * tl.stride_b + c * 16u, tl.lds + blk * 1024u);
+    lds_dma_16(tl.base, min(max(r, tl.rmin), tl.rmax) * tl.stride_b + c * 16u, tl.lds + blk * 1024u);
   }
 }
 
@@ -309,6 +314,11 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     }
     if (tok_a < p.causal_rows && p.extra_lo < p.t_all) hi_max = p.t_all;
     if (row0 + kBlockM > p.rows_total) hi_min = 0;  // ragged tile: always take the masked path
+    // all four are the same in every lane; say so, so that they live in scalar registers
+    lo_min = __builtin_amdgcn_readfirstlane(lo_min);
+    lo_max = __builtin_amdgcn_readfirstlane(lo_max);
+    hi_min = __builtin_amdgcn_readfirstlane(hi_min);
+    hi_max = __builtin_amdgcn_readfirstlane(hi_max);
   }
   const uint32_t split_begin = p.tile_first + split * p.tiles_per_split;
   const uint32_t split_end = min(split_begin + p.tiles_per_split, p.tile_end);
@@ -426,10 +436,10 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     const uint32_t t_last = (te - 1u) * kBlockN;
     const uint32_t ld_rot = (mt * (L::NBLK >= 32 ? 2u : 1u)) & (uint32_t)(L::NBLK - 1);
     auto k_load = [&](uint32_t t0, lds_char* buf) {
-      return make_tile_load(kbase, kstride_b, min(t0, t_last), p.t_all, p.ring_mask, buf, ld_rot);
+      return make_tile_load(kbase, kstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, ld_rot);
     };
     auto v_load = [&](uint32_t t0, lds_char* buf) {
-      return make_tile_load(vbase, vstride_b, min(t0, t_last), p.t_all, p.ring_mask, buf, ld_rot);
+      return make_tile_load(vbase, vstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, ld_rot);
     };
 
     issue_tile<D, false>(k_load(tb * kBlockN, k0), wave, lane);
