@@ -28,8 +28,19 @@
 // below 65504.
 #include "attn_params.h"
 
+#include <type_traits>
+
 namespace dg {
 namespace {
+
+// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N)
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -81,6 +92,30 @@ __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
 }
 
 // two floats -> packed pair of E (round to nearest even), low half = a
+// Score MFMAs, written as assembly so that their accumulator is an ordinary VGPR tuple.  O fills
+// all 256 accumulation registers at head_dim 512; the compiler gives every MFMA of such a
+// kernel an accumulation-register destination, which made it park one block of O in VGPRs
+// around each tile's score MFMAs (48 register moves per tile and wave).
+// The compiler does not know these are MFMAs, so the one hazard it would otherwise cover is
+// handled here: mfma_scores_done() must separate the last score MFMA from the first
+// non-MFMA read of the scores.  Back-to-back MFMAs that accumulate into the same registers need
+// no wait states, and operands that come from LDS are covered by the s_waitcnt the compiler
+// inserts for the asm operands.
+template <bool F16>
+__device__ __forceinline__ void mfma_scores_first(f32x16& s, u32x4 a, u32x4 b) {
+  if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
+}
+template <bool F16>
+__device__ __forceinline__ void mfma_scores_acc(f32x16& s, u32x4 a, u32x4 b) {
+  if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
+}
+// 24 wait states: more than the 20 a 16-pass MFMA result needs before a VALU may read it
+__device__ __forceinline__ void mfma_scores_done(f32x16& s) {
+  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s));
+}
+
 template <bool F16>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
   if constexpr (F16) {
@@ -185,62 +220,83 @@ struct TileLoad {
   uint32_t stride_b;  // bytes between key rows in global memory
   uint32_t rmin;      // first row of the tile that may be read
   uint32_t rmax;      // last row of the tile that may be read
-  uint32_t lds;       // LDS byte address of the destination buffer
-  uint32_t rot;       // rotation of the order in which the tile's KiB blocks are fetched
+  uint32_t lds;       // LDS byte address of the destination buffer (padded layout: of this wave's first row)
+  // padded layout only, per lane: byte offsets from base of this lane's chunk in the first and
+  // the last row that may be read, and in the row of this wave's load 0
+  uint32_t lo_l, hi_l, raw0;
 };
 
+template <int D, bool IS_V>
 __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_t tok_stride_b, uint32_t t0,
                                                    uint32_t t_min, uint32_t t_all, uint32_t ring_mask, lds_char* buf,
-                                                   uint32_t rot) {
+                                                   uint32_t wave, uint32_t lane) {
+  using L = Lay<D>;
   TileLoad tl;
   tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
   tl.stride_b = (uint32_t)tok_stride_b;
   tl.rmin = t_min > t0 ? t_min - t0 : 0u;
   tl.rmax = t_all - 1u - t0;
   tl.lds = (uint32_t)(size_t)buf;
-  tl.rot = rot;
+  if constexpr (L::PAD) {
+    tl.lds += wave * (IS_V ? L::V_STRIDE : L::K_STRIDE);
+    tl.lo_l = tl.rmin * tl.stride_b + lane * 16u;
+    tl.hi_l = tl.rmax * tl.stride_b + lane * 16u;
+    tl.raw0 = wave * tl.stride_b + lane * 16u;
+  }
   return tl;
 }
 
-// The load is written as assembly on purpose: the compiler orders every LDS read after a
+// The loads are written as assembly on purpose: the compiler orders every LDS read after a
 // direct-to-LDS load it knows about with s_waitcnt vmcnt(0), which would expose the whole
-// fetch latency once per tile.  The kernel waits for these loads itself, at the top of the
-// tile loop, one iteration after they were issued.
-__device__ __forceinline__ void lds_dma_16(const char* base_uniform, uint32_t voff, uint32_t lds_dst_uniform) {
-  // all scalar operands are wave-uniform by construction; readfirstlane tells the compiler so
-  // (it returns a signed int: without the casts the low half would be sign-extended over the
-  // high half)
-  const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_dst_uniform);
+// fetch latency once per tile.  The kernel waits for these loads itself (wait_vmem_but).
+// All scalar operands are wave-uniform by construction; readfirstlane tells the compiler so
+// (it returns a signed int: without the casts the low half of the address would be
+// sign-extended over the high half).
+__device__ __forceinline__ uint64_t uniform_address(const char* base_uniform) {
   const uint64_t b = (uint64_t)base_uniform;
-  const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32) |
-                        (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base)
-               : "memory");
+  return ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32) |
+         (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
 }
-
-template <int D, bool IS_V>
-__device__ __forceinline__ void issue_tile_part(const TileLoad& tl, int k, uint32_t wave, uint32_t lane) {
-  using L = Lay<D>;
-  if (L::NBLK < 4 && k * 4 + wave >= (uint32_t)L::NBLK) return;
-  // Workgroups that stream the same keys run in near lockstep; each starts its tile at a
-  // different block so that they do not all ask the L2 for the same lines at the same time.
-  const uint32_t blk = (k * 4 + wave + tl.rot) & (uint32_t)(L::NBLK - 1);
-  if constexpr (L::PAD) {
-    // one instruction = one key row: the row part of the address is scalar
-    const char* row = tl.base + (uint64_t)min(max(blk, tl.rmin), tl.rmax) * tl.stride_b;
-    lds_dma_16(row, lane * 16u, tl.lds + blk * (IS_V ? L::V_STRIDE : L::K_STRIDE));
+// lane l: 16 bytes from base + voff -> LDS byte (lds_dst + LDS_IMM) + 16 * l
+template <int LDS_IMM>
+__device__ __forceinline__ void lds_dma_16(const char* base_uniform, uint32_t voff, uint32_t lds_dst_uniform) {
+  const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_dst_uniform);
+  const uint64_t base = uniform_address(base_uniform);
+  if constexpr (LDS_IMM == 0) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base)
+                 : "memory");
   } else {
-    const uint32_t pch = blk * 64 + lane;
-    const uint32_t r = pch / L::CPR, pc = pch % L::CPR;
-    const uint32_t c = pc ^ (IS_V ? L::swz_v(r) : L::swz_k(r));
-    lds_dma_16(tl.base, min(max(r, tl.rmin), tl.rmax) * tl.stride_b + c * 16u, tl.lds + blk * 1024u);
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff),
+                 "s"(base), "n"(LDS_IMM)
+                 : "memory", "scc");
   }
 }
 
-template <int D, bool IS_V>
+template <int D, bool IS_V, int K>
+__device__ __forceinline__ void issue_tile_part(const TileLoad& tl, uint32_t wave, uint32_t lane) {
+  using L = Lay<D>;
+  if (L::NBLK < 4 && K * 4 + wave >= (uint32_t)L::NBLK) return;
+  if constexpr (L::PAD) {
+    // one instruction = one key row (row 4 K + wave): everything but the clamp of the row is
+    // either per tile or a compile-time constant
+    uint32_t voff;
+    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(voff) : "v"(tl.raw0 + (uint32_t)(4 * K) * tl.stride_b), "v"(tl.lo_l), "v"(tl.hi_l));
+    lds_dma_16<4 * K * (IS_V ? L::V_STRIDE : L::K_STRIDE)>(tl.base, voff, tl.lds);
+  } else {
+    const uint32_t blk = K * 4 + wave;
+    const uint32_t pch = blk * 64 + lane;
+    const uint32_t r = pch / L::CPR, pc = pch % L::CPR;
+    const uint32_t c = pc ^ (IS_V ? L::swz_v(r) : L::swz_k(r));
+    lds_dma_16<0>(tl.base, min(max(r, tl.rmin), tl.rmax) * tl.stride_b + c * 16u, tl.lds + blk * 1024u);
+  }
+}
+
+template <int D, bool IS_V, int K = 0>
 __device__ __forceinline__ void issue_tile(const TileLoad& tl, uint32_t wave, uint32_t lane) {
-#pragma unroll
-  for (int k = 0; k < Lay<D>::NLD; ++k) issue_tile_part<D, IS_V>(tl, k, wave, lane);
+  if constexpr (K < Lay<D>::NLD) {
+    issue_tile_part<D, IS_V, K>(tl, wave, lane);
+    issue_tile<D, IS_V, K + 1>(tl, wave, lane);
+  }
 }
 
 // PIPE: issue Q.K^T of tile j+1 before the softmax of tile j (needs a second score tile in
@@ -272,10 +328,14 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const uint32_t nstream = p.hkv * p.n_splits;
   const uint32_t wg = blockIdx.x;
   const uint32_t slot_in_xcd = wg >> 3;
-  const uint32_t stream = (slot_in_xcd / p.n_mtiles) * 8u + (wg & 7u);
-  const uint32_t mt = slot_in_xcd % p.n_mtiles;
+  // (the divisions by run-time values are done by the vector unit; readfirstlane tells the
+  // compiler the results are the same in every lane, so everything derived from them stays in
+  // scalar registers)
+  const uint32_t stream = __builtin_amdgcn_readfirstlane((slot_in_xcd / p.n_mtiles) * 8u + (wg & 7u));
+  const uint32_t mt = __builtin_amdgcn_readfirstlane(slot_in_xcd % p.n_mtiles);
   if (stream >= nstream) return;
-  const uint32_t kvh = stream / p.n_splits, split = stream % p.n_splits;
+  const uint32_t kvh = __builtin_amdgcn_readfirstlane(stream / p.n_splits);
+  const uint32_t split = __builtin_amdgcn_readfirstlane(stream % p.n_splits);
 
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -322,8 +382,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   }
   const uint32_t split_begin = p.tile_first + split * p.tiles_per_split;
   const uint32_t split_end = min(split_begin + p.tiles_per_split, p.tile_end);
-  const uint32_t tb = max(lo_min / kBlockN, split_begin);
-  const uint32_t te = min((hi_max + kBlockN - 1) / kBlockN, split_end);
+  const uint32_t tb = __builtin_amdgcn_readfirstlane(max(lo_min / kBlockN, split_begin));
+  const uint32_t te = __builtin_amdgcn_readfirstlane(min((hi_max + kBlockN - 1) / kBlockN, split_end));
   const uint32_t ntile = te > tb ? te - tb : 0u;
 
   // ---- Q fragments: B operand of S^T = K.Q^T, lane = row, 8 consecutive d per step ----
@@ -408,19 +468,20 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   // scheduling barriers keep that interleaving.
   auto qk_tile = [&](lds_char* kb, const TileLoad& next_k, uint32_t ld_lane, bool with_loads) -> f32x16 {
     f32x16 s;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) s[e] = 0.f;
     u32x4 kf[PFK];
 #pragma unroll
     for (int i = 0; i < PFK; ++i) kf[i] = k_frag(kb, i);
-#pragma unroll
-    for (int st = 0; st < NQK; ++st) {
+    static_for<0, NQK>([&](auto st_c) {
+      constexpr int st = decltype(st_c)::value;
       __builtin_amdgcn_sched_barrier(0);
-      s = mfma16<F16>(kf[st % PFK], qf[st], s);
-      if (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
-      if (with_loads && st % LDK_EVERY == 0 && st / LDK_EVERY < NLD)
-        issue_tile_part<D, false>(next_k, st / LDK_EVERY, wave, ld_lane);
-    }
+      if constexpr (st == 0) mfma_scores_first<F16>(s, kf[0], qf[0]);
+      else mfma_scores_acc<F16>(s, kf[st % PFK], qf[st]);
+      if constexpr (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
+      if constexpr (st % LDK_EVERY == 0 && st / LDK_EVERY < NLD) {
+        if (with_loads) issue_tile_part<D, false, st / LDK_EVERY>(next_k, wave, ld_lane);
+      }
+    });
+    mfma_scores_done(s);
     __builtin_amdgcn_sched_barrier(0);
     return s;
   };
@@ -434,23 +495,22 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     // Loads for a tile past the last one are not branched around: they fetch the last tile
     // again into a buffer nobody reads any more.
     const uint32_t t_last = (te - 1u) * kBlockN;
-    const uint32_t ld_rot = (mt * (L::NBLK >= 32 ? 2u : 1u)) & (uint32_t)(L::NBLK - 1);
-    auto k_load = [&](uint32_t t0, lds_char* buf) {
-      return make_tile_load(kbase, kstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, ld_rot);
+    auto k_load = [&](uint32_t t0, lds_char* buf, uint32_t ln) {
+      return make_tile_load<D, false>(kbase, kstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, wave, ln);
     };
-    auto v_load = [&](uint32_t t0, lds_char* buf) {
-      return make_tile_load(vbase, vstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, ld_rot);
+    auto v_load = [&](uint32_t t0, lds_char* buf, uint32_t ln) {
+      return make_tile_load<D, true>(vbase, vstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, wave, ln);
     };
 
-    issue_tile<D, false>(k_load(tb * kBlockN, k0), wave, lane);
-    if constexpr (PIPE) issue_tile<D, false>(k_load((tb + 1) * kBlockN, k1), wave, lane);
-    issue_tile<D, true>(v_load(tb * kBlockN, v0), wave, lane);
+    issue_tile<D, false>(k_load(tb * kBlockN, k0, lane), wave, lane);
+    if constexpr (PIPE) issue_tile<D, false>(k_load((tb + 1) * kBlockN, k1, lane), wave, lane);
+    issue_tile<D, true>(v_load(tb * kBlockN, v0, lane), wave, lane);
     wait_vmem_all();
     __syncthreads();
     f32x16 s_cur;
     if constexpr (PIPE) {
       // K(tb+2) goes where K(tb) sits, so it cannot be issued before this first tile is consumed
-      s_cur = qk_tile(k0, k_load(0, k0), lane, false);
+      s_cur = qk_tile(k0, k_load(0, k0, lane), lane, false);
     }
     DG_PHASE(0)
 
@@ -475,8 +535,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       asm volatile("" : "+v"(lane_l));
       // PIPE: K(jj) was consumed one iteration ago, its buffer takes K(jj+2).
       // otherwise: K(jj+1) goes to the other buffer while K(jj) is read.
-      const TileLoad next_k = PIPE ? k_load(t0 + 2 * kBlockN, kb_even) : k_load(t0 + kBlockN, kb_odd);
-      const TileLoad next_v = v_load(t0 + kBlockN, vb_free);
+      const TileLoad next_k = PIPE ? k_load(t0 + 2 * kBlockN, kb_even, lane_l) : k_load(t0 + kBlockN, kb_odd, lane_l);
+      const TileLoad next_v = v_load(t0 + kBlockN, vb_free, lane_l);
       f32x16 s_next;
       if constexpr (PIPE) {
         if (jj + 1 < ntile) s_next = qk_tile(kb_odd, next_k, lane_l, true);
@@ -576,19 +636,18 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         u32x4 va[PFV + 1];
 #pragma unroll
         for (int f = 0; f <= PFV; ++f) va[f] = v_frag_n(f);
-#pragma unroll
-        for (int f = 0; f < NVF; ++f) {
-          const int ks = f / NDBW, i = f % NDBW;
-#pragma unroll
-          for (int j = 0; j < NRBW; ++j) {
-            const int n = f * NRBW + j;   // MFMA index within the tile
+        static_for<0, NVF>([&](auto f_c) {
+          constexpr int f = decltype(f_c)::value, ks = f / NDBW, i = f % NDBW;
+          static_for<0, NRBW>([&](auto j_c) {
+            constexpr int j = decltype(j_c)::value, n = f * NRBW + j;   // n: MFMA index within the tile
             __builtin_amdgcn_sched_barrier(0);
             o[i * NRBW + j] = mfma16<F16>(va[f % (PFV + 1)], pbv[j], o[i * NRBW + j]);
-            if (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
-            if (n % LDV_EVERY == 0 && n / LDV_EVERY < NLD) issue_tile_part<D, true>(next_v, n / LDV_EVERY, wave, lane_l);
-          }
-          if (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
-        }
+            if constexpr (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
+            if constexpr (n % LDV_EVERY == 0 && n / LDV_EVERY < NLD)
+              issue_tile_part<D, true, n / LDV_EVERY>(next_v, wave, lane_l);
+          });
+          if constexpr (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
+        });
         __builtin_amdgcn_sched_barrier(0);
       }
 #ifdef DG_ATTN_PHASE_TIMING
