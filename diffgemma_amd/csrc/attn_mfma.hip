@@ -17,8 +17,19 @@
 // waves would read the whole V tile through it; with the d split each V fragment is read once
 // per workgroup and the small P tile is what gets read four times.
 //
-// K and V tiles arrive by 16-byte direct-to-LDS loads, double buffered, issued one instruction
-// at a time between MFMAs.  The running max is only raised (and O rescaled) when some row's
+// The tile loop is software-pipelined with one barrier per tile.  One wave per SIMD issues in
+// order, so anything that is to overlap the matrix pipe has to sit between MFMAs in program
+// order.  For tile j a wave issues, in this order:
+//   score MFMAs of tile j+1, the softmax of tile j spread between them (its scores were
+//   accumulated one tile earlier), ending with the store of P(j);
+//   [barrier, waiting first for this wave's loads of V(j) and K(j+2)]
+//   the first LDS reads of the P.V phase, then the last few score MFMAs of tile j+1, whose K
+//   fragments were already in registers (they cover the latency of those reads);
+//   the P.V MFMAs of tile j with, spread between them, the global loads of V(j+1) and K(j+3),
+//   the copy of tile j+1's scores and the first K fragment reads of tile j+2.
+// K and V tiles arrive by 16-byte direct-to-LDS loads into two buffers each; P, the rescale
+// factors and the flags are double buffered too, which is what makes one barrier enough.
+// The running max is only raised (and O rescaled) when some row's
 // tile max exceeds it by more than 2^tau; the raise is broadcast to the d owners through LDS
 // together with P.  Rescaling O costs about as much as the tile's P.V MFMAs, and with unit-RMS
 // Q and K and no 1/sqrt(d) the scores of a row spread over tens of log2 units, so a small tau
@@ -97,8 +108,8 @@ __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
 // kernel an accumulation-register destination, which made it park one block of O in VGPRs
 // around each tile's score MFMAs (48 register moves per tile and wave).
 // The compiler does not know these are MFMAs, so the one hazard it would otherwise cover is
-// handled here: mfma_scores_done() must separate the last score MFMA from the first
-// non-MFMA read of the scores.  Back-to-back MFMAs that accumulate into the same registers need
+// handled here: the last score MFMA of a tile (mfma_scores_last) is followed by the wait
+// states a non-MFMA read of the scores needs.  Back-to-back MFMAs that accumulate into the same registers need
 // no wait states, and operands that come from LDS are covered by the s_waitcnt the compiler
 // inserts for the asm operands.
 template <bool F16>
@@ -111,9 +122,42 @@ __device__ __forceinline__ void mfma_scores_acc(f32x16& s, u32x4 a, u32x4 b) {
   if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
   else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
 }
-// 24 wait states: more than the 20 a 16-pass MFMA result needs before a VALU may read it
-__device__ __forceinline__ void mfma_scores_done(f32x16& s) {
-  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(s));
+// Last score MFMA of a tile, followed by 24 wait states: more than the 20 a 16-pass MFMA result
+// needs before a VALU may read it.  They are part of the same asm statement so that no
+// compiler-made register copy of the scores can land between the MFMA and the wait.
+template <bool F16>
+__device__ __forceinline__ void mfma_scores_last(f32x16& s, u32x4 a, u32x4 b) {
+  if constexpr (F16)
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
+  else
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
+}
+
+// x *= c for a value that lives in an accumulation register, without the register allocator
+// moving it into the VGPR class
+__device__ __forceinline__ float scale_acc(float x, float c) {
+  float tmp;
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+               : "+a"(x), "=&v"(tmp)
+               : "v"(c));
+  return x;
+}
+// dst = src for a score tile, as instructions the compiler cannot move or merge away; part I of
+// 8 copies elements 2 I and 2 I + 1
+template <int I>
+__device__ __forceinline__ void copy_scores_part(f32x16& dst, const f32x16& src) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  f32x2 d;
+  const f32x2 v = {src[2 * I], src[2 * I + 1]};
+  asm volatile("v_mov_b64 %0, %1" : "=v"(d) : "v"(v));
+  dst[2 * I] = d[0];
+  dst[2 * I + 1] = d[1];
+}
+// the value, made opaque to the optimiser (so that what is derived from it is recomputed where
+// it is used instead of being kept in registers across the tile loop)
+__device__ __forceinline__ uint32_t opaque(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
 }
 
 template <bool F16>
@@ -299,9 +343,7 @@ __device__ __forceinline__ void issue_tile(const TileLoad& tl, uint32_t wave, ui
   }
 }
 
-// PIPE: issue Q.K^T of tile j+1 before the softmax of tile j (needs a second score tile in
-// registers; used where the register file has room for it).
-template <int D, bool F16, bool PIPE>
+template <int D, bool F16>
 __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   using L = Lay<D>;
   constexpr int NSTEP = D / 16, NDB = D / 32;
@@ -313,13 +355,15 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   // One LDS block, carved by hand so that the order of the buffers is fixed:
   //   K0 K1 | V0 V1 | P: [ks][row-block][lane] x 16 B | per-row rescale factor of this tile |
   //   "row-block raised its max this tile" flags | epilogue (m, l) per row
+  // P, the rescale factors and the flags exist twice (tiles alternate), which is what lets the
+  // tile loop run with a single barrier per tile.
   constexpr int OFF_K0 = 0, OFF_K1 = L::K_BYTES, OFF_V0 = 2 * L::K_BYTES, OFF_V1 = OFF_V0 + L::V_BYTES;
-  constexpr int OFF_P = 2 * L::K_BYTES + 2 * L::V_BYTES, OFF_CORR = OFF_P + 2 * 4 * 1024;
-  constexpr int OFF_FLAG = OFF_CORR + 4 * 32 * 4, OFF_ML = OFF_FLAG + 16, LDS_BYTES = OFF_ML + 4 * 32 * 2 * 4;
+  constexpr int P_BYTES = 2 * 4 * 1024, CORR_BYTES = 4 * 32 * 4, FLAG_BYTES = 16;
+  constexpr int OFF_P = 2 * L::K_BYTES + 2 * L::V_BYTES, OFF_CORR = OFF_P + 2 * P_BYTES;
+  constexpr int OFF_FLAG = OFF_CORR + 2 * CORR_BYTES, OFF_ML = OFF_FLAG + 2 * FLAG_BYTES;
+  constexpr int LDS_BYTES = OFF_ML + 4 * 32 * 2 * 4;
   static_assert(L::K_BYTES % 16 == 0 && L::V_BYTES % 16 == 0, "buffer alignment");
   __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
-  float* const scorr = (float*)(smem + OFF_CORR);
-  uint32_t* const sflag = (uint32_t*)(smem + OFF_FLAG);
   float* const sml = (float*)(smem + OFF_ML);
 
   // ---- which (KV head, split, row tile) this workgroup owns ----
@@ -414,7 +458,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[i][e] = 0.f;
   float m_ref = -INFINITY;  // running reference max, log2 units (scale folded in)
-  float l_part = 0.f;       // this lane's share of the row sum (its 16 of every 32 keys)
+  float l_part = 0.f;       // this lane's share of the row sum (its 16 of every 32 keys),
+  float l_part2 = 0.f;      // kept as two partial sums
 
   const char* kbase = (const char*)p.k + (int64_t)kvh * p.k_head_stride * 2;
   const char* vbase = (const char*)p.v + (int64_t)kvh * p.v_head_stride * 2;
@@ -428,12 +473,12 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const uint32_t v_swz = L::swz_v(v_row);
   const uint32_t v_lane_chunk = 2u * h16 + ((i16 & 3u) >> 1);
   const uint32_t v_lane_off = v_row * L::V_STRIDE + (i16 & 1u) * 8u + (L::PAD ? v_lane_chunk * 16u : 0u);
-  lds_char* const pbuf = (lds_char*)(smem + OFF_P);
 
   constexpr int NLD = L::NLD;                    // load instructions per wave, tile and matrix
   constexpr int NQK = NSTEP, NPV = 2 * NACC;     // MFMAs per wave and tile in each phase
-  constexpr int PFK = NQK < 8 ? NQK : 8;         // K fragment reads kept in flight ahead of the MFMAs
-  constexpr int LDK_EVERY = NQK / NLD, LDV_EVERY = NPV / NLD;
+  constexpr int PFK = NQK < 4 ? NQK : 4;         // K fragment reads kept in flight ahead of the MFMAs
+  constexpr int LD_EVERY = NPV / (2 * NLD);      // P.V MFMAs per tile load instruction
+  static_assert(LD_EVERY >= 1 && 2 * NLD * LD_EVERY <= NPV, "tile loads must fit between the P.V MFMAs");
 
   // K fragment of MFMA step st: A operand, lane = key row l32, 8 consecutive d at 16*st + 8*g2
   auto k_frag = [&](lds_char* kb, int st) -> u32x4 {
@@ -459,32 +504,6 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vb + off + 8 * L::V_STRIDE)));
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
-  auto p_frag = [&](int ks, uint32_t rbk) -> u32x4 {
-    return *(lds_u32x4*)(pbuf + (((uint32_t)ks * 4u + rbk) * 64u + lane) * 16u);
-  };
-
-  // S^T = K.Q^T for one tile.  PFK fragment reads run ahead of the MFMA that consumes them and
-  // the next K tile's global loads are issued one instruction every LDK_EVERY MFMAs; the
-  // scheduling barriers keep that interleaving.
-  auto qk_tile = [&](lds_char* kb, const TileLoad& next_k, uint32_t ld_lane, bool with_loads) -> f32x16 {
-    f32x16 s;
-    u32x4 kf[PFK];
-#pragma unroll
-    for (int i = 0; i < PFK; ++i) kf[i] = k_frag(kb, i);
-    static_for<0, NQK>([&](auto st_c) {
-      constexpr int st = decltype(st_c)::value;
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (st == 0) mfma_scores_first<F16>(s, kf[0], qf[0]);
-      else mfma_scores_acc<F16>(s, kf[st % PFK], qf[st]);
-      if constexpr (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
-      if constexpr (st % LDK_EVERY == 0 && st / LDK_EVERY < NLD) {
-        if (with_loads) issue_tile_part<D, false, st / LDK_EVERY>(next_k, wave, ld_lane);
-      }
-    });
-    mfma_scores_done(s);
-    __builtin_amdgcn_sched_barrier(0);
-    return s;
-  };
 
   DG_PHASE_DECL
   if (ntile > 0) {
@@ -493,7 +512,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     lds_char* const v0 = (lds_char*)(smem + OFF_V0);
     lds_char* const v1 = (lds_char*)(smem + OFF_V1);
     // Loads for a tile past the last one are not branched around: they fetch the last tile
-    // again into a buffer nobody reads any more.
+    // again into a buffer nobody reads any more (or whose scores nobody uses).
     const uint32_t t_last = (te - 1u) * kBlockN;
     auto k_load = [&](uint32_t t0, lds_char* buf, uint32_t ln) {
       return make_tile_load<D, false>(kbase, kstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, wave, ln);
@@ -502,170 +521,237 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       return make_tile_load<D, true>(vbase, vstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, wave, ln);
     };
 
+    // ---- softmax of one tile, cut into NCH pieces ----
+    // The pieces of tile jj run between the score MFMAs of tile jj+1: one wave per SIMD issues
+    // in order, so vector work only overlaps the matrix pipe if it sits between MFMAs in
+    // program order.  A vector instruction that needs the result of the one before it waits
+    // about 8 cycles, an independent one issues after 4, so every piece is written as a group of
+    // independent operations (four scores at a time, two partial row sums).
+    // State that lives across pieces:
+    float tmax = 0.f, m_use = 0.f;
+    float ex[4] = {0.f, 0.f, 0.f, 0.f};
+    u32x4 pk4 = {0, 0, 0, 0};
+    auto softmax_piece = [&](auto c_c, f32x16& s, uint32_t t0, uint32_t par) {
+      constexpr int c = decltype(c_c)::value;
+      if constexpr (c == 0) {
+        // mask (edge tiles only)
+        const bool masked = !(t0 >= lo_max && t0 + kBlockN <= hi_min);
+        if (masked) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const uint32_t t = t0 + 8u * (e >> 2) + 4u * g2 + (e & 3);
+            if (!key_visible(rb, t, p.t_all)) s[e] = -INFINITY;
+          }
+        }
+      } else if constexpr (c == 1) {
+        // tile max of the row, as a tree
+        const float a0 = fmaxf(fmaxf(s[0], s[1]), s[2]), a1 = fmaxf(fmaxf(s[3], s[4]), s[5]);
+        const float a2 = fmaxf(fmaxf(s[6], s[7]), s[8]), a3 = fmaxf(fmaxf(s[9], s[10]), s[11]);
+        const float a4 = fmaxf(fmaxf(s[12], s[13]), s[14]);
+        tmax = fmaxf(fmaxf(fmaxf(a0, a1), a2), fmaxf(fmaxf(a3, a4), s[15]));
+      } else if constexpr (c == 2) {
+        // online softmax with a lazily raised reference max
+        tmax = max_across_halves(tmax) * p.scale_log2;
+        const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau<F16>) != 0ull;
+        bool rescale = false;   // some row of the block has accumulated something that changes
+        if (raise) {
+          const float m_new = fmaxf(m_ref, tmax);
+          const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+          rescale = __builtin_amdgcn_ballot_w64(m_ref != -INFINITY && corr != 1.f) != 0ull;
+          l_part *= corr;
+          l_part2 *= corr;
+          // the d owners rescale O after the barrier
+          if (g2 == 0) ((float*)(smem + OFF_CORR + par * CORR_BYTES))[wave * 32u + l32] = corr;
+          m_ref = m_new;
+        }
+        if (lane == 0) ((uint32_t*)(smem + OFF_FLAG + par * FLAG_BYTES))[wave] = rescale ? 1u : 0u;
+        m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+      } else {
+        // scores 4 q .. 4 q + 3 in two steps: (a) scale and subtract, first two exponentials;
+        // (b) the other two exponentials, rounding to the MFMA operand type, and for every
+        // second q the store of a k-step's B operand and its share of the row sum
+        constexpr int q = (c - 3) / 2;
+        if constexpr ((c - 3) % 2 == 0) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ex[i] = __builtin_fmaf(s[4 * q + i], p.scale_log2, -m_use);
+          ex[0] = __builtin_amdgcn_exp2f(ex[0]);
+          ex[1] = __builtin_amdgcn_exp2f(ex[1]);
+        } else {
+          ex[2] = __builtin_amdgcn_exp2f(ex[2]);
+          ex[3] = __builtin_amdgcn_exp2f(ex[3]);
+          pk4[(2 * q) % 4] = pack2<F16>(ex[0], ex[1]);
+          pk4[(2 * q + 1) % 4] = pack2<F16>(ex[2], ex[3]);
+          if constexpr (q % 2 == 1) {
+            // register image of the B operand of MFMA k-step q/2 for (row l32, lane half g2)
+            *(lds_u32x4*)((lds_char*)(smem + OFF_P) + par * P_BYTES + (((uint32_t)(q / 2) * 4u + wave) * 64u + lane) * 16u) =
+                pk4;
+            // the row sum uses the rounded probabilities, the same numbers P.V multiplies
+            l_part = add_pair<F16>(pk4[0], l_part);
+            l_part2 = add_pair<F16>(pk4[1], l_part2);
+            l_part = add_pair<F16>(pk4[2], l_part);
+            l_part2 = add_pair<F16>(pk4[3], l_part2);
+          }
+        }
+      }
+    };
+    constexpr int NCH = 3 + 8;   // pieces the softmax of a tile is cut into
+
+    // S^T = K.Q^T, MFMA steps [ST0, ST1) of the tile in kb.  The K fragments of steps
+    // 0 .. PFK-1 are already in (or on their way to) kf; fragment reads run PFK ahead of the
+    // MFMA that consumes them.  With SOFTMAX, the softmax of the previous tile (scores in
+    // s_prev) is spread over the steps below NSPLIT.  The scheduling barriers keep the
+    // interleaving as written.
+    constexpr int NSPLIT = NQK - PFK;   // steps before the tile's barrier; the rest need no more LDS reads
+    u32x4 kf[PFK];
+    auto kf_preload = [&](lds_char* kb) {
+#pragma unroll
+      for (int i = 0; i < PFK; ++i) kf[i] = k_frag(kb, i);
+    };
+    auto qk_steps = [&](auto st0_c, auto st1_c, lds_char* kb, auto softmax_c, auto wait_c, f32x16& s, f32x16& s_prev,
+                        uint32_t t0_prev, uint32_t par) {
+      constexpr bool SOFTMAX = decltype(softmax_c)::value, WAIT = decltype(wait_c)::value;
+      static_for<decltype(st0_c)::value, decltype(st1_c)::value>([&](auto st_c) {
+        constexpr int st = decltype(st_c)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (st == 0) mfma_scores_first<F16>(s, kf[0], qf[0]);
+        else if constexpr (WAIT && st == NQK - 1) mfma_scores_last<F16>(s, kf[st % PFK], qf[st]);
+        else mfma_scores_acc<F16>(s, kf[st % PFK], qf[st]);
+        if constexpr (st + PFK < NQK) kf[st % PFK] = k_frag(kb, st + PFK);
+        if constexpr (SOFTMAX && st < NSPLIT) {
+          // pieces [st NCH / NSPLIT, (st+1) NCH / NSPLIT) follow MFMA st
+          static_for<st * NCH / (NSPLIT > 0 ? NSPLIT : 1), (st + 1) * NCH / (NSPLIT > 0 ? NSPLIT : 1)>(
+              [&](auto c_c) { softmax_piece(c_c, s_prev, t0_prev, par); });
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using ISPLIT = std::integral_constant<int, NSPLIT>;
+    using IQK = std::integral_constant<int, NQK>;
+
     issue_tile<D, false>(k_load(tb * kBlockN, k0, lane), wave, lane);
-    if constexpr (PIPE) issue_tile<D, false>(k_load((tb + 1) * kBlockN, k1, lane), wave, lane);
+    issue_tile<D, false>(k_load((tb + 1) * kBlockN, k1, lane), wave, lane);
     issue_tile<D, true>(v_load(tb * kBlockN, v0, lane), wave, lane);
     wait_vmem_all();
     __syncthreads();
-    f32x16 s_cur;
-    if constexpr (PIPE) {
-      // K(tb+2) goes where K(tb) sits, so it cannot be issued before this first tile is consumed
-      s_cur = qk_tile(k0, k_load(0, k0, lane), lane, false);
-    }
+    // s_a: scores of the tile whose softmax is due; s_b: scores being accumulated for the next.
+    // s_b is copied into s_a during each tile's P.V by copy_scores_part(), not by an assignment:
+    // the compiler would merge the two and place its own copy right behind (or before) the last
+    // score MFMA, reading the registers before the MFMA has written them.
+    f32x16 s_a, s_b;
+    kf_preload(k0);
+    qk_steps(I0{}, IQK{}, k0, std::false_type{}, std::true_type{}, s_a, s_b, 0u, 0u);
+    __syncthreads();   // every wave is done with K(tb): its buffer takes K(tb+2)
+    issue_tile<D, false>(k_load((tb + 2) * kBlockN, k0, lane), wave, lane);
+    kf_preload(k1);
     DG_PHASE(0)
 
     for (uint32_t jj = 0; jj < ntile; ++jj) {
+      const uint32_t par = jj & 1u;
       const uint32_t t0 = (tb + jj) * kBlockN;
-      lds_char* const kb_even = (jj & 1u) ? k1 : k0;   // holds K(jj)
-      lds_char* const kb_odd = (jj & 1u) ? k0 : k1;    // holds K(jj+1) (PIPE) or takes it
-      lds_char* const vb_cur = (jj & 1u) ? v1 : v0;    // holds V(jj)
-      lds_char* const vb_free = (jj & 1u) ? v0 : v1;   // refill with V(jj+1)
+      lds_char* const kb_next = par ? k0 : k1;    // holds K(jj+1); takes K(jj+3) after the barrier
+      lds_char* const kb_next2 = par ? k1 : k0;   // holds K(jj+2) once the barrier is passed
+      lds_char* const vb_cur = par ? v1 : v0;     // holds V(jj)
+      lds_char* const vb_free = par ? v0 : v1;    // takes V(jj+1)
 
-      // Barrier A: the K tile this iteration multiplies has landed everywhere (this wave's share
-      // of it is older than its NLD loads of V(jj), which may still be in flight), and every wave
-      // is done with the previous tile (its K/V buffers, the P tile and the rescale words can be
-      // reused).
-      wait_vmem_but<NLD>();
-      DG_PHASE(1)
-      __syncthreads();
-      DG_PHASE(2)
-      // Re-derive the per-lane global offsets of the tile loads inside every iteration: hoisted
-      // out of the loop they would cost more live VGPRs than this kernel has.
-      uint32_t lane_l = lane;
-      asm volatile("" : "+v"(lane_l));
-      // PIPE: K(jj) was consumed one iteration ago, its buffer takes K(jj+2).
-      // otherwise: K(jj+1) goes to the other buffer while K(jj) is read.
-      const TileLoad next_k = PIPE ? k_load(t0 + 2 * kBlockN, kb_even, lane_l) : k_load(t0 + kBlockN, kb_odd, lane_l);
-      const TileLoad next_v = v_load(t0 + kBlockN, vb_free, lane_l);
-      f32x16 s_next;
-      if constexpr (PIPE) {
-        if (jj + 1 < ntile) s_next = qk_tile(kb_odd, next_k, lane_l, true);
-      } else {
-        s_cur = qk_tile(kb_even, next_k, lane_l, true);
-      }
-#ifdef DG_ATTN_PHASE_TIMING
-      asm volatile("s_nop 0" ::"v"(s_cur[0]), "v"(s_cur[15]));  // the scores have to exist before the clock is read
-#endif
+      // ---- row-owner role: scores of the next tile, softmax of this one ----
+      // (K(jj+1) has landed everywhere: its loads were waited for before the previous barrier,
+      // and its first fragments were read during the previous tile's P.V.  For the last tile
+      // the "next" scores are those of a repeated tile and go unused.)
+      if constexpr (NSPLIT == 0)
+        static_for<0, NCH>([&](auto c_c) { softmax_piece(c_c, s_a, t0, par); });
+      qk_steps(I0{}, ISPLIT{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par);
       DG_PHASE(3)
-
-      // ---- mask (edge tiles only) ----
-      const bool masked = !(t0 >= lo_max && t0 + kBlockN <= hi_min);
-      if (masked) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const uint32_t t = t0 + 8u * (e >> 2) + 4u * g2 + (e & 3);
-          if (!key_visible(rb, t, p.t_all)) s_cur[e] = -INFINITY;
-        }
-      }
-      // ---- online softmax with a lazily raised reference max ----
-      float tmax = s_cur[0];
-#pragma unroll
-      for (int e = 1; e < 16; ++e) tmax = fmaxf(tmax, s_cur[e]);
-      tmax = max_across_halves(tmax) * p.scale_log2;
-      const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau<F16>) != 0ull;
-      if (raise) {
-        const float m_new = fmaxf(m_ref, tmax);
-        const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
-        l_part *= corr;
-        if (g2 == 0) scorr[wave * 32u + l32] = corr;   // the d owners rescale O after barrier B
-        m_ref = m_new;
-      }
-      if (lane == 0) sflag[wave] = raise ? 1u : 0u;
-      const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        u32x4 pk4;
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-          const int e = 8 * ks + j;
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e], p.scale_log2, -m_use));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e + 1], p.scale_log2, -m_use));
-          const uint32_t pk = pack2<F16>(p0, p1);
-          pk4[j >> 1] = pk;
-          // the row sum uses the rounded probabilities, the same numbers P.V multiplies
-          l_part = add_pair<F16>(pk, l_part);
-        }
-        // register image of the B operand of MFMA k-step ks for (row l32, lane half g2)
-        *(lds_u32x4*)(pbuf + (((uint32_t)ks * 4u + wave) * 64u + lane) * 16u) = pk4;
-      }
+      // The one barrier of the tile.  Before it: this wave's loads of V(jj) and K(jj+2), issued
+      // during the previous tile's P.V, have landed, its P is written and the last K fragments
+      // of the tile are in registers (the barrier's fence waits for all three).  After it: P,
+      // the rescale words and V(jj) of this tile are visible to the d owners; every wave is done
+      // reading K(jj+1), V(jj-1) and the previous tile's P (which has its own buffer), so their
+      // buffers can be refilled.
+      wait_vmem_all();
       DG_PHASE(4)
-      // Barrier B: P and the rescale words of this tile are visible to the d owners, and V(jj)
-      // has landed everywhere (only the NLD loads of the next K tile, issued after it, may still
-      // be in flight).
-      wait_vmem_but<NLD>();
       __syncthreads();
       DG_PHASE(5)
 
       // ---- d-owner role ----
-      {
-        const u32x4 fl = *(lds_u32x4*)((lds_char*)sflag);
-        if (__builtin_amdgcn_readfirstlane(fl[0] | fl[1] | fl[2] | fl[3]) != 0u) {
-          // O lives in accumulator registers, which only MFMA and the accvgpr moves can touch.
-          // Spelling the multiply out keeps the values in that register class on both sides of
-          // this rarely taken branch; a plain `o[i] *= corr` makes the allocator shuttle all of
-          // O through VGPRs and spill.
+      lds_char* const pbuf = (lds_char*)(smem + OFF_P) + par * P_BYTES;
+      auto p_frag = [&](int ks, uint32_t rbk) -> u32x4 {
+        return *(lds_u32x4*)(pbuf + (((uint32_t)ks * 4u + rbk) * 64u + lane) * 16u);
+      };
+      constexpr int NVF = 2 * NDBW;                    // V^T fragments per tile and wave
+      constexpr int PFV = NVF - 1 < 3 ? NVF - 1 : 3;   // fragment reads in flight ahead of the MFMAs
+      auto v_frag_n = [&](int f) { return v_frag(vb_cur, f / NDBW, dgrp * NDBW + f % NDBW); };
+      // first reads of the P.V phase; the last score MFMAs of the next tile cover their latency
+      const u32x4 fl = *(lds_u32x4*)((lds_char*)(smem + OFF_FLAG) + par * FLAG_BYTES);
+      u32x4 pbv[NRBW];
 #pragma unroll
-          for (int j = 0; j < NRBW; ++j) {
-            const uint32_t rbk = rgrp * NRBW + j;
-            if (__builtin_amdgcn_readfirstlane(fl[rbk]) == 0u) continue;
-            const float corr = scorr[rbk * 32u + l32];
+      for (int j = 0; j < NRBW; ++j) pbv[j] = p_frag(0, rgrp * NRBW + j);
+      u32x4 va[PFV + 1];
 #pragma unroll
-            for (int i = 0; i < NDBW; ++i)
+      for (int f = 0; f <= PFV; ++f) va[f] = v_frag_n(f);
+      qk_steps(ISPLIT{}, IQK{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par);
+
+      // Re-derive the per-lane global offsets of the tile loads inside every iteration: hoisted
+      // out of the loop they would cost more live VGPRs than this kernel has.
+      const uint32_t lane_l = opaque(lane);
+      const TileLoad next_v = v_load(t0 + kBlockN, vb_free, lane_l);
+      const TileLoad next_k = k_load(t0 + 3 * kBlockN, kb_next, lane_l);
+      if (__builtin_amdgcn_readfirstlane(fl[0] | fl[1] | fl[2] | fl[3]) != 0u) {
+        // O lives in accumulator registers, which only MFMA and the accvgpr moves can touch.
+        // Spelling the multiply out keeps the values in that register class on both sides of
+        // this rarely taken branch; a plain `o[i] *= corr` makes the allocator shuttle all of
+        // O through VGPRs and spill.
+        const float* const scorr = (const float*)(smem + OFF_CORR + par * CORR_BYTES);
 #pragma unroll
-              for (int e = 0; e < 16; ++e) {
-                float tmp;
-                float x = o[i * NRBW + j][e];
-                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
-                             : "+a"(x), "=&v"(tmp)
-                             : "v"(corr));
-                o[i * NRBW + j][e] = x;
-              }
-          }
+        for (int j = 0; j < NRBW; ++j) {
+          const uint32_t rbk = rgrp * NRBW + j;
+          if (__builtin_amdgcn_readfirstlane(fl[rbk]) == 0u) continue;
+          const float corr = scorr[rbk * 32u + l32];
+#pragma unroll
+          for (int i = 0; i < NDBW; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[i * NRBW + j][e] = scale_acc(o[i * NRBW + j][e], corr);
         }
-        // O^T += V^T . P^T: per k-step, NDBW V^T fragments x NRBW P fragments.  The P fragments
-        // of a k-step stay in registers for the whole step; V^T fragments are fetched PFV ahead
-        // of the one that multiplies, and each P fragment of k-step 1 replaces its k-step 0
-        // counterpart right after that one's last use.  V(jj+1)'s global loads are spread between
-        // the MFMAs.
-        constexpr int NVF = 2 * NDBW;                    // V^T fragments per tile and wave
-        constexpr int PFV = NVF - 1 < 3 ? NVF - 1 : 3;   // fragment reads in flight ahead of the MFMAs
-        auto v_frag_n = [&](int f) { return v_frag(vb_cur, f / NDBW, dgrp * NDBW + f % NDBW); };
-        u32x4 pbv[NRBW];
-#pragma unroll
-        for (int j = 0; j < NRBW; ++j) pbv[j] = p_frag(0, rgrp * NRBW + j);
-        u32x4 va[PFV + 1];
-#pragma unroll
-        for (int f = 0; f <= PFV; ++f) va[f] = v_frag_n(f);
-        static_for<0, NVF>([&](auto f_c) {
-          constexpr int f = decltype(f_c)::value, ks = f / NDBW, i = f % NDBW;
-          static_for<0, NRBW>([&](auto j_c) {
-            constexpr int j = decltype(j_c)::value, n = f * NRBW + j;   // n: MFMA index within the tile
-            __builtin_amdgcn_sched_barrier(0);
-            o[i * NRBW + j] = mfma16<F16>(va[f % (PFV + 1)], pbv[j], o[i * NRBW + j]);
-            if constexpr (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
-            if constexpr (n % LDV_EVERY == 0 && n / LDV_EVERY < NLD)
-              issue_tile_part<D, true, n / LDV_EVERY>(next_v, wave, lane_l);
-          });
-          if constexpr (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
-        });
-        __builtin_amdgcn_sched_barrier(0);
       }
+      // O^T += V^T . P^T: per k-step, NDBW V^T fragments x NRBW P fragments.  The P fragments
+      // of a k-step stay in registers for the whole step; V^T fragments are fetched PFV ahead
+      // of the one that multiplies, and each P fragment of k-step 1 replaces its k-step 0
+      // counterpart right after that one's last use.  Spread between the MFMAs: the global
+      // loads of V(jj+1) and K(jj+3), alternating; the copy of the next tile's scores to where
+      // the softmax expects them; at the end, the first K fragments of tile jj+2.
+      constexpr int COPY_AT = NPV >= 16 ? NPV / 2 : 0;   // MFMA index after which the copy starts
+      static_for<0, NVF>([&](auto f_c) {
+        constexpr int f = decltype(f_c)::value, ks = f / NDBW, i = f % NDBW;
+        static_for<0, NRBW>([&](auto j_c) {
+          constexpr int j = decltype(j_c)::value, n = f * NRBW + j;   // n: MFMA index within the tile
+          __builtin_amdgcn_sched_barrier(0);
+          o[i * NRBW + j] = mfma16<F16>(va[f % (PFV + 1)], pbv[j], o[i * NRBW + j]);
+          if constexpr (ks == 0 && i == NDBW - 1) pbv[j] = p_frag(1, rgrp * NRBW + j);
+          if constexpr (n % LD_EVERY == 0 && n / LD_EVERY < 2 * NLD) {
+            constexpr int q = n / LD_EVERY;
+            if constexpr (q % 2 == 0) issue_tile_part<D, true, q / 2>(next_v, wave, lane_l);
+            else issue_tile_part<D, false, q / 2>(next_k, wave, lane_l);
+          }
+          if constexpr (NPV >= 16 && n >= COPY_AT && n < COPY_AT + 8) copy_scores_part<n - COPY_AT>(s_a, s_b);
+        });
+        if constexpr (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (NPV < 16) static_for<0, 8>([&](auto i_c) { copy_scores_part<decltype(i_c)::value>(s_a, s_b); });
+      kf_preload(kb_next2);
 #ifdef DG_ATTN_PHASE_TIMING
-      asm volatile("s_nop 0" ::"a"(o[0][0]), "a"(o[NACC - 1][15]));
+      o[0][0] = scale_acc(o[0][0], 1.f);   // the accumulators have to exist before the clock is read
 #endif
       DG_PHASE(6)
-      if constexpr (PIPE) {
-        if (jj + 1 < ntile) s_cur = s_next;
-      }
     }
-    // the loads issued for the tile after the last one must not outlive this workgroup's LDS
+    // the loads issued for tiles after the last one must not outlive this workgroup's LDS
     wait_vmem_all();
   }
 
   // ---- epilogue ----
   DG_PHASE_STORE
   // row owners publish (m, l) of their rows; d owners normalise and store their slice of O
-  const float l_tot = sum_across_halves(l_part);
+  const float l_tot = sum_across_halves(l_part + l_part2);
   __syncthreads();   // the last tile's readers are done with LDS
   if (g2 == 0) {
     sml[(wave * 32u + l32) * 2u] = m_ref;
@@ -734,8 +820,7 @@ template <int D, bool F16>
 hipError_t launch_one(const AttnParams& p, hipStream_t s) {
   const uint32_t nstream = p.hkv * p.n_splits;
   const uint32_t grid = ((nstream + 7u) / 8u) * p.n_mtiles * 8u;
-  constexpr bool kPipe = D < 512;  // at D=512 the second score tile does not fit next to O and Q
-  hipLaunchKernelGGL((attn_mfma_kernel<D, F16, kPipe>), dim3(grid), dim3(256), 0, s, p);
+  hipLaunchKernelGGL((attn_mfma_kernel<D, F16>), dim3(grid), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 
