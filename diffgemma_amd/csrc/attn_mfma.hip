@@ -35,7 +35,7 @@
 // Q and K and no 1/sqrt(d) the scores of a row spread over tens of log2 units, so a small tau
 // would rescale some row block on almost every tile.  Any reference below the true max is
 // exact as long as nothing overflows: P <= 2^tau, and the fp32 sums stay below
-// 2^tau * keys * |v|, far from 2^127 for tau = 64.  With f16 operands P itself has to stay
+// 2^tau * keys * |v|, far from 2^127 for tau = 80.  With f16 operands P itself has to stay
 // below 65504.
 #include "attn_params.h"
 
@@ -69,7 +69,7 @@ typedef __attribute__((address_space(3))) void lds_void;
 
 // log2 units by which a tile max may exceed the reference max before the reference is raised
 template <bool F16>
-constexpr float kTau = F16 ? 12.0f : 64.0f;
+constexpr float kTau = F16 ? 12.0f : 80.0f;
 
 // Optional per-phase cycle accounting (development builds only): every wave sums the cycles
 // it spends in each phase of the tile loop and stores the sums at the end.
@@ -133,15 +133,24 @@ __device__ __forceinline__ void mfma_scores_last(f32x16& s, u32x4 a, u32x4 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
 }
 
-// x *= c for a value that lives in an accumulation register, without the register allocator
-// moving it into the VGPR class
-__device__ __forceinline__ float scale_acc(float x, float c) {
-  float tmp;
-  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
-               : "+a"(x), "=&v"(tmp)
-               : "v"(c));
+// x *= c for values that live in accumulation registers, without the register allocator moving
+// them into the VGPR class.  Four at a time, so that no instruction waits for the one before it.
+__device__ __forceinline__ void scale_acc4(float& x0, float& x1, float& x2, float& x3, float c) {
+  float t0, t1, t2, t3;
+  asm volatile(
+      "v_accvgpr_read_b32 %4, %0\n\tv_accvgpr_read_b32 %5, %1\n\tv_accvgpr_read_b32 %6, %2\n\tv_accvgpr_read_b32 %7, %3\n\t"
+      "v_mul_f32 %4, %4, %8\n\tv_mul_f32 %5, %5, %8\n\tv_mul_f32 %6, %6, %8\n\tv_mul_f32 %7, %7, %8\n\t"
+      "v_accvgpr_write_b32 %0, %4\n\tv_accvgpr_write_b32 %1, %5\n\tv_accvgpr_write_b32 %2, %6\n\tv_accvgpr_write_b32 %3, %7\n\t"
+      "s_nop 3"   // the compiler does not see these writes: keep a following MFMA clear of them
+      : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+      : "v"(c));
+}
+#ifdef DG_ATTN_PHASE_TIMING
+__device__ __forceinline__ float touch_acc(float x) {
+  asm volatile("s_nop 0" : "+a"(x));
   return x;
 }
+#endif
 // dst = src for a score tile, as instructions the compiler cannot move or merge away; part I of
 // 8 copies elements 2 I and 2 I + 1
 template <int I>
@@ -152,6 +161,10 @@ __device__ __forceinline__ void copy_scores_part(f32x16& dst, const f32x16& src)
   asm volatile("v_mov_b64 %0, %1" : "=v"(d) : "v"(v));
   dst[2 * I] = d[0];
   dst[2 * I + 1] = d[1];
+}
+__device__ __forceinline__ u32x4 opaque4(u32x4 v) {
+  asm volatile("" : "+v"(v));
+  return v;
 }
 // the value, made opaque to the optimiser (so that what is derived from it is recomputed where
 // it is used instead of being kept in registers across the tile loop)
@@ -287,6 +300,20 @@ __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_
     tl.hi_l = tl.rmax * tl.stride_b + lane * 16u;
     tl.raw0 = wave * tl.stride_b + lane * 16u;
   }
+  return tl;
+}
+
+// The descriptor with every field computed at this point of the program (the compiler would
+// otherwise sink the arithmetic to the first use, which sits behind a branch where nothing
+// overlaps it).
+__device__ __forceinline__ TileLoad pinned(TileLoad tl) {
+  uint64_t b = (uint64_t)tl.base;
+  uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+  uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  uint32_t lds = (uint32_t)__builtin_amdgcn_readfirstlane(tl.lds);
+  asm volatile("" : "+s"(lo), "+s"(hi), "+s"(lds), "+v"(tl.lo_l), "+v"(tl.hi_l), "+v"(tl.raw0));
+  tl.base = (const char*)(((uint64_t)hi << 32) | lo);
+  tl.lds = lds;
   return tl;
 }
 
@@ -536,7 +563,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       if constexpr (c == 0) {
         // mask (edge tiles only)
         const bool masked = !(t0 >= lo_max && t0 + kBlockN <= hi_min);
-        if (masked) {
+        if (__builtin_expect(masked, 0)) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const uint32_t t = t0 + 8u * (e >> 2) + 4u * g2 + (e & 3);
@@ -554,7 +581,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         tmax = max_across_halves(tmax) * p.scale_log2;
         const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau<F16>) != 0ull;
         bool rescale = false;   // some row of the block has accumulated something that changes
-        if (raise) {
+        if (__builtin_expect(raise, 0)) {
           const float m_new = fmaxf(m_ref, tmax);
           const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
           rescale = __builtin_amdgcn_ballot_w64(m_ref != -INFINITY && corr != 1.f) != 0ull;
@@ -608,7 +635,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       for (int i = 0; i < PFK; ++i) kf[i] = k_frag(kb, i);
     };
     auto qk_steps = [&](auto st0_c, auto st1_c, lds_char* kb, auto softmax_c, auto wait_c, f32x16& s, f32x16& s_prev,
-                        uint32_t t0_prev, uint32_t par) {
+                        uint32_t t0_prev, uint32_t par, auto&& after) {
       constexpr bool SOFTMAX = decltype(softmax_c)::value, WAIT = decltype(wait_c)::value;
       static_for<decltype(st0_c)::value, decltype(st1_c)::value>([&](auto st_c) {
         constexpr int st = decltype(st_c)::value;
@@ -620,8 +647,10 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         if constexpr (SOFTMAX && st < NSPLIT) {
           // pieces [st NCH / NSPLIT, (st+1) NCH / NSPLIT) follow MFMA st
           static_for<st * NCH / (NSPLIT > 0 ? NSPLIT : 1), (st + 1) * NCH / (NSPLIT > 0 ? NSPLIT : 1)>(
-              [&](auto c_c) { softmax_piece(c_c, s_prev, t0_prev, par); });
+              [&](auto c_c) {
+                softmax_piece(c_c, s_prev, t0_prev, par); });
         }
+        after(st_c);
       });
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -640,7 +669,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     // score MFMA, reading the registers before the MFMA has written them.
     f32x16 s_a, s_b;
     kf_preload(k0);
-    qk_steps(I0{}, IQK{}, k0, std::false_type{}, std::true_type{}, s_a, s_b, 0u, 0u);
+    auto nothing = [](auto) {};
+    qk_steps(I0{}, IQK{}, k0, std::false_type{}, std::true_type{}, s_a, s_b, 0u, 0u, nothing);
     __syncthreads();   // every wave is done with K(tb): its buffer takes K(tb+2)
     issue_tile<D, false>(k_load((tb + 2) * kBlockN, k0, lane), wave, lane);
     kf_preload(k1);
@@ -660,7 +690,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // the "next" scores are those of a repeated tile and go unused.)
       if constexpr (NSPLIT == 0)
         static_for<0, NCH>([&](auto c_c) { softmax_piece(c_c, s_a, t0, par); });
-      qk_steps(I0{}, ISPLIT{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par);
+      qk_steps(I0{}, ISPLIT{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par, nothing);
       DG_PHASE(3)
       // The one barrier of the tile.  Before it: this wave's loads of V(jj) and K(jj+2), issued
       // during the previous tile's P.V, have landed, its P is written and the last K fragments
@@ -682,21 +712,28 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       constexpr int PFV = NVF - 1 < 3 ? NVF - 1 : 3;   // fragment reads in flight ahead of the MFMAs
       auto v_frag_n = [&](int f) { return v_frag(vb_cur, f / NDBW, dgrp * NDBW + f % NDBW); };
       // first reads of the P.V phase; the last score MFMAs of the next tile cover their latency
-      const u32x4 fl = *(lds_u32x4*)((lds_char*)(smem + OFF_FLAG) + par * FLAG_BYTES);
+      u32x4 fl = *(lds_u32x4*)((lds_char*)(smem + OFF_FLAG) + par * FLAG_BYTES);
       u32x4 pbv[NRBW];
 #pragma unroll
       for (int j = 0; j < NRBW; ++j) pbv[j] = p_frag(0, rgrp * NRBW + j);
       u32x4 va[PFV + 1];
 #pragma unroll
       for (int f = 0; f <= PFV; ++f) va[f] = v_frag_n(f);
-      qk_steps(ISPLIT{}, IQK{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par);
-
-      // Re-derive the per-lane global offsets of the tile loads inside every iteration: hoisted
-      // out of the loop they would cost more live VGPRs than this kernel has.
+      // The descriptors of this tile's global loads are worked out between those MFMAs, not
+      // behind the branch below, where nothing would overlap them.  The per-lane offsets are
+      // re-derived in every iteration: hoisted out of the loop they would cost more live VGPRs
+      // than this kernel has.
       const uint32_t lane_l = opaque(lane);
-      const TileLoad next_v = v_load(t0 + kBlockN, vb_free, lane_l);
-      const TileLoad next_k = k_load(t0 + 3 * kBlockN, kb_next, lane_l);
-      if (__builtin_amdgcn_readfirstlane(fl[0] | fl[1] | fl[2] | fl[3]) != 0u) {
+      TileLoad next_v, next_k;
+      qk_steps(ISPLIT{}, IQK{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par, [&](auto st_c) {
+        constexpr int st = decltype(st_c)::value;
+        if constexpr (st == NSPLIT) next_v = pinned(v_load(t0 + kBlockN, vb_free, lane_l));
+        if constexpr (st == (NSPLIT + 1 < NQK ? NSPLIT + 1 : NSPLIT))
+          next_k = pinned(k_load(t0 + 3 * kBlockN, kb_next, lane_l));
+      });
+      // keep every use of the flags behind those MFMAs: they are what hides the latency of the read
+      fl = opaque4(fl);
+      if (__builtin_expect(__builtin_amdgcn_readfirstlane(fl[0] | fl[1] | fl[2] | fl[3]) != 0u, 0)) {
         // O lives in accumulator registers, which only MFMA and the accvgpr moves can touch.
         // Spelling the multiply out keeps the values in that register class on both sides of
         // this rarely taken branch; a plain `o[i] *= corr` makes the allocator shuttle all of
@@ -710,7 +747,15 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
           for (int i = 0; i < NDBW; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o[i * NRBW + j][e] = scale_acc(o[i * NRBW + j][e], corr);
+            for (int e = 0; e < 16; e += 4) {
+              f32x16& a = o[i * NRBW + j];
+              float x0 = a[e], x1 = a[e + 1], x2 = a[e + 2], x3 = a[e + 3];
+              scale_acc4(x0, x1, x2, x3, corr);
+              a[e] = x0;
+              a[e + 1] = x1;
+              a[e + 2] = x2;
+              a[e + 3] = x3;
+            }
         }
       }
       // O^T += V^T . P^T: per k-step, NDBW V^T fragments x NRBW P fragments.  The P fragments
@@ -718,7 +763,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // of the one that multiplies, and each P fragment of k-step 1 replaces its k-step 0
       // counterpart right after that one's last use.  Spread between the MFMAs: the global
       // loads of V(jj+1) and K(jj+3), alternating; the copy of the next tile's scores to where
-      // the softmax expects them; at the end, the first K fragments of tile jj+2.
+      // the softmax expects them; behind the last MFMAs, the reads of the first K fragments of
+      // tile jj+2 (pinned there: at the loop end the compiler would move them to the top of the
+      // next iteration, in front of the MFMAs that wait for them).
       constexpr int COPY_AT = NPV >= 16 ? NPV / 2 : 0;   // MFMA index after which the copy starts
       static_for<0, NVF>([&](auto f_c) {
         constexpr int f = decltype(f_c)::value, ks = f / NDBW, i = f % NDBW;
@@ -733,14 +780,15 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
             else issue_tile_part<D, false, q / 2>(next_k, wave, lane_l);
           }
           if constexpr (NPV >= 16 && n >= COPY_AT && n < COPY_AT + 8) copy_scores_part<n - COPY_AT>(s_a, s_b);
+          if constexpr (NPV >= PFK && n >= NPV - PFK) kf[n - (NPV - PFK)] = k_frag(kb_next2, n - (NPV - PFK));
         });
         if constexpr (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
       });
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (NPV < 16) static_for<0, 8>([&](auto i_c) { copy_scores_part<decltype(i_c)::value>(s_a, s_b); });
-      kf_preload(kb_next2);
+      if constexpr (NPV < PFK) kf_preload(kb_next2);
 #ifdef DG_ATTN_PHASE_TIMING
-      o[0][0] = scale_acc(o[0][0], 1.f);   // the accumulators have to exist before the clock is read
+      o[0][0] = touch_acc(o[0][0]);   // the accumulators have to exist before the clock is read
 #endif
       DG_PHASE(6)
     }
