@@ -95,6 +95,10 @@ __global__ void __launch_bounds__(64) attn_scalar_kernel(const AttnParams p, con
 }
 
 // One wave per stacked row: combines the per-split (m, l, O) triples.
+// The split weights are worked out first (they are the same for the whole row); the O partials
+// are then streamed with four splits' loads in flight per lane, which is what lets the kernel
+// run at memory speed: the partials of a 32k-prefix global layer are tens of megabytes.
+static_assert(kMaxSplits <= 64, "one lane per split");
 __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, const uint32_t hd) {
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t gr = blockIdx.x * 4 + wave;  // global stacked row over all KV heads
@@ -103,31 +107,54 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
   const uint32_t tok = r / p.group, qh = kvh * p.group + r % p.group;
   const size_t split_stride = (size_t)p.hkv * p.rows_pad;
   const size_t row = (size_t)kvh * p.rows_pad + r;
-  float mx = -INFINITY;
-  for (uint32_t s = 0; s < p.n_splits; ++s) mx = fmaxf(mx, p.part_ml[(s * split_stride + row) * 2]);
-  float den = 0.f;
-  for (uint32_t s = 0; s < p.n_splits; ++s) {
-    const float ms = p.part_ml[(s * split_stride + row) * 2], ls = p.part_ml[(s * split_stride + row) * 2 + 1];
-    if (ls > 0.f) den += ls * exp2f(ms - mx);
+  // lane s holds split s's (m, l); the row's weights come from wave reductions
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < p.n_splits) {
+    const float2 ml = *(const float2*)(p.part_ml + ((size_t)lane * split_stride + row) * 2);
+    ms = ml.x;
+    ls = ml.y;
   }
+  float mx = ms;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  float wl = ls > 0.f ? ls * exp2f(ms - mx) : 0.f;   // l_s * 2^(m_s - m)
+  const float den = wave_sum(wl);
   const float inv = den > 0.f ? 1.f / den : 0.f;
+  const float w_mine = ls > 0.f ? exp2f(ms - mx) * inv : 0.f;   // weight of split `lane`
   const size_t ooff = ((size_t)tok * p.hq + qh) * hd;
+  const float* const base = p.part_o + row * hd;
+  const size_t sstride = split_stride * hd;
   for (uint32_t d4 = lane; d4 < hd / 4; d4 += 64) {
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t s = 0; s < p.n_splits; ++s) {
-      const float ms = p.part_ml[(s * split_stride + row) * 2], ls = p.part_ml[(s * split_stride + row) * 2 + 1];
-      if (!(ls > 0.f)) continue;
-      const float w = exp2f(ms - mx);
-      const float4 a = ((const float4*)(p.part_o + (s * split_stride + row) * hd))[d4];
+    uint32_t s = 0;
+    for (; s + 4 <= p.n_splits; s += 4) {
+      const float4 a0 = ((const float4*)(base + (s + 0) * sstride))[d4];
+      const float4 a1 = ((const float4*)(base + (s + 1) * sstride))[d4];
+      const float4 a2 = ((const float4*)(base + (s + 2) * sstride))[d4];
+      const float4 a3 = ((const float4*)(base + (s + 3) * sstride))[d4];
+      const float w0 = __shfl(w_mine, s + 0, 64), w1 = __shfl(w_mine, s + 1, 64);
+      const float w2 = __shfl(w_mine, s + 2, 64), w3 = __shfl(w_mine, s + 3, 64);
+      o.x += w0 * a0.x + w1 * a1.x + w2 * a2.x + w3 * a3.x;
+      o.y += w0 * a0.y + w1 * a1.y + w2 * a2.y + w3 * a3.y;
+      o.z += w0 * a0.z + w1 * a1.z + w2 * a2.z + w3 * a3.z;
+      o.w += w0 * a0.w + w1 * a1.w + w2 * a2.w + w3 * a3.w;
+    }
+    for (; s < p.n_splits; ++s) {
+      const float4 a = ((const float4*)(base + s * sstride))[d4];
+      const float w = __shfl(w_mine, s, 64);
       o.x += w * a.x;
       o.y += w * a.y;
       o.z += w * a.z;
       o.w += w * a.w;
     }
-    store_out(p, ooff + d4 * 4 + 0, o.x * inv);
-    store_out(p, ooff + d4 * 4 + 1, o.y * inv);
-    store_out(p, ooff + d4 * 4 + 2, o.z * inv);
-    store_out(p, ooff + d4 * 4 + 3, o.w * inv);
+    if (p.out_dtype == DT_F32) {
+      ((float4*)((float*)p.out + ooff))[d4] = o;
+    } else {
+      store_out(p, ooff + d4 * 4 + 0, o.x);
+      store_out(p, ooff + d4 * 4 + 1, o.y);
+      store_out(p, ooff + d4 * 4 + 2, o.z);
+      store_out(p, ooff + d4 * 4 + 3, o.w);
+    }
   }
   if (lane == 0) {
     if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));

@@ -8,6 +8,7 @@ namespace dg {
 
 enum : uint32_t { DT_BF16 = 0, DT_F16 = 1, DT_F32 = 2 };
 
+constexpr uint32_t kMaxSplits = 64;   // key-range splits per launch: the merge gives each a lane
 constexpr int kBlockM = 128;   // stacked query rows per workgroup (4 waves x 32)
 constexpr int kBlockN = 32;    // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;

@@ -13,7 +13,7 @@
 
 namespace {
 
-constexpr uint32_t kMaxSplits = 64;
+using dg::kMaxSplits;
 constexpr size_t kAlign = 256;
 
 inline size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
