@@ -283,7 +283,8 @@ struct TileLoad {
   uint32_t lo_l, hi_l, raw0;
 };
 
-template <int D, bool IS_V>
+// FIRST: the tile may begin before t_min (only the first tile a workgroup visits can).
+template <int D, bool IS_V, bool FIRST>
 __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_t tok_stride_b, uint32_t t0,
                                                    uint32_t t_min, uint32_t t_all, uint32_t ring_mask, lds_char* buf,
                                                    uint32_t wave, uint32_t lane) {
@@ -291,8 +292,8 @@ __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_
   TileLoad tl;
   tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
   tl.stride_b = (uint32_t)tok_stride_b;
-  tl.rmin = t_min > t0 ? t_min - t0 : 0u;
-  tl.rmax = t_all - 1u - t0;
+  tl.rmin = FIRST && t_min > t0 ? t_min - t0 : 0u;
+  tl.rmax = min(t_all - 1u - t0, (uint32_t)kBlockN - 1u);
   tl.lds = (uint32_t)(size_t)buf;
   if constexpr (L::PAD) {
     tl.lds += wave * (IS_V ? L::V_STRIDE : L::K_STRIDE);
@@ -541,11 +542,18 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     // Loads for a tile past the last one are not branched around: they fetch the last tile
     // again into a buffer nobody reads any more (or whose scores nobody uses).
     const uint32_t t_last = (te - 1u) * kBlockN;
+    // (in the loop only tiles behind the workgroup's first one are loaded)
     auto k_load = [&](uint32_t t0, lds_char* buf, uint32_t ln) {
-      return make_tile_load<D, false>(kbase, kstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, wave, ln);
+      return make_tile_load<D, false, false>(kbase, kstride_b, min(t0, t_last), 0u, p.t_all, p.ring_mask, buf, wave, ln);
     };
     auto v_load = [&](uint32_t t0, lds_char* buf, uint32_t ln) {
-      return make_tile_load<D, true>(vbase, vstride_b, min(t0, t_last), lo_min, p.t_all, p.ring_mask, buf, wave, ln);
+      return make_tile_load<D, true, false>(vbase, vstride_b, min(t0, t_last), 0u, p.t_all, p.ring_mask, buf, wave, ln);
+    };
+    auto k_load_first = [&](lds_char* buf) {
+      return make_tile_load<D, false, true>(kbase, kstride_b, tb * kBlockN, lo_min, p.t_all, p.ring_mask, buf, wave, lane);
+    };
+    auto v_load_first = [&](lds_char* buf) {
+      return make_tile_load<D, true, true>(vbase, vstride_b, tb * kBlockN, lo_min, p.t_all, p.ring_mask, buf, wave, lane);
     };
 
     // ---- softmax of one tile, cut into NCH pieces ----
@@ -658,9 +666,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     using ISPLIT = std::integral_constant<int, NSPLIT>;
     using IQK = std::integral_constant<int, NQK>;
 
-    issue_tile<D, false>(k_load(tb * kBlockN, k0, lane), wave, lane);
+    issue_tile<D, false>(k_load_first(k0), wave, lane);
     issue_tile<D, false>(k_load((tb + 1) * kBlockN, k1, lane), wave, lane);
-    issue_tile<D, true>(v_load(tb * kBlockN, v0, lane), wave, lane);
+    issue_tile<D, true>(v_load_first(v0), wave, lane);
     wait_vmem_all();
     __syncthreads();
     // s_a: scores of the tile whose softmax is due; s_b: scores being accumulated for the next.
@@ -766,6 +774,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // the softmax expects them; behind the last MFMAs, the reads of the first K fragments of
       // tile jj+2 (pinned there: at the loop end the compiler would move them to the top of the
       // next iteration, in front of the MFMAs that wait for them).
+#ifdef DG_FINE_PHASES
+      DG_PHASE(1)
+#endif
       constexpr int COPY_AT = NPV >= 16 ? NPV / 2 : 0;   // MFMA index after which the copy starts
       static_for<0, NVF>([&](auto f_c) {
         constexpr int f = decltype(f_c)::value, ks = f / NDBW, i = f % NDBW;
