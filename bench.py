@@ -9,6 +9,7 @@ batch already resident in HBM.  Prints ONE JSON line.
 from __future__ import annotations
 
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -134,14 +135,36 @@ def main():
         A.forward(desc, qd, kd, out, lse, ws)
     torch.cuda.synchronize()
     capi.prof_begin(args.steps)
+    round_len = max(1, min(50, args.steps // 4))
+    marks = [torch.cuda.Event(enable_timing=True)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         A.forward(desc, qd, kd, out, lse, ws)
+        if (i + 1) % round_len == 0:      # an event per round, on the stream the library launches on
+            marks.append(torch.cuda.Event(enable_timing=True))
+            marks[-1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     kern_ms_total, n_rec = capi.prof_end()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     kern_ms = kern_ms_total / max(n_rec, 1)
+    round_ms = sorted(marks[i].elapsed_time(marks[i + 1]) / round_len for i in range(len(marks) - 1))
+    rounds = {"steps_per_round": round_len, "n": len(round_ms), "min_ms_per_step": round_ms[0],
+              "median_ms_per_step": round_ms[len(round_ms) // 2]} if round_ms else None
+
+    # ---- what nothing but MFMAs sustains on this machine, right after the timed steps ----
+    lib = capi.load()
+    sink = torch.zeros(256 * 256, dtype=torch.float32, device="cuda")
+    mf = C.c_uint64(0)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for rep in range(2):                   # first pass warms the code up
+        e0.record()
+        for _ in range(8):
+            capi.check(lib.dg_calib_mfma(sink.data_ptr(), sink.numel() * 4, 256, 1000, C.byref(mf), A.stream_handle()))
+        e1.record()
+        torch.cuda.synchronize()
+    mfma_only_tflops = 8 * mf.value / (e0.elapsed_time(e1) * 1e-3) / 1e12
 
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kern_tflops = flops / (kern_ms * 1e-3) / 1e12
@@ -164,8 +187,10 @@ def main():
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": kern_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
                      "kernel": "attn_mfma_kernel", "kernel_ms": kern_ms,
+                     "mfma_only_microkernel_tflops": mfma_only_tflops,
+                     "frac_of_mfma_only_microkernel": kern_tflops / mfma_only_tflops,
                      "kv_gbs": kv_bytes / (kern_ms * 1e-3) / 1e9, "hbm_peak_gbs": PEAK_HBM_GBS},
-        "check": check, "input_gen_s": t_gen,
+        "rounds": rounds, "check": check, "input_gen_s": t_gen,
     }
     if not args.no_cpu_baseline:
         # per-row FLOPs (rows differ under the causal part of the mask)

@@ -24,7 +24,7 @@ EXPORTS = (
     "dg_attn_resolved_splits", "dg_attn_forward", "dg_attn_strerror", "dg_attn_abi_version",
     "dg_attn_visible_pairs", "dg_attention_dispatch", "dg_attention_state_bytes", "dg_kv_row_bytes",
     "dg_kv_region_bytes", "dg_kv_slot", "dg_layer_kv_slots", "dg_prof_begin", "dg_prof_end",
-    "dg_calib_copy",
+    "dg_calib_copy", "dg_calib_mfma",
 )
 
 
@@ -125,6 +125,8 @@ def load():
     lib.dg_layer_kv_slots.restype = C.c_uint64
     lib.dg_calib_copy.argtypes = [VP, VP, C.c_size_t, VP]
     lib.dg_calib_copy.restype = C.c_int
+    lib.dg_calib_mfma.argtypes = [VP, C.c_size_t, C.c_uint32, C.c_uint32, P(C.c_uint64), VP]
+    lib.dg_calib_mfma.restype = C.c_int
     lib.dg_prof_begin.argtypes = [C.c_uint32]
     lib.dg_prof_begin.restype = C.c_int
     lib.dg_prof_end.argtypes = [P(C.c_double), P(C.c_uint32)]

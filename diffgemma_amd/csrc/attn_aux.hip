@@ -197,7 +197,42 @@ __global__ void calib_copy_kernel(const uint4* __restrict__ src, uint4* __restri
     dst[i] = src[i];
 }
 
+// Nothing but MFMAs: four independent 32x32x16 bf16 accumulators per wave, one wave per SIMD.
+// What this sustains is the ceiling the attention kernel's MFMA rate is compared with on the
+// machine at hand (the published peak assumes the maximum clock).
+typedef float calib_f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 calib_bf16x8 __attribute__((ext_vector_type(8)));
+__global__ void __launch_bounds__(256) calib_mfma_kernel(float* sink, uint32_t iters) {
+  calib_bf16x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (__bf16)(1.0f + 0.001f * (float)((threadIdx.x + i) & 7));
+    b[i] = (__bf16)(0.5f - 0.001f * (float)((threadIdx.x * 3 + i) & 7));
+  }
+  calib_f32x16 c0, c1, c2, c3;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) c0[e] = c1[e] = c2[e] = c3[e] = 0.f;
+  for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+    }
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc += c0[e] + c1[e] + c2[e] + c3[e];
+  if (acc == 123.456f) sink[blockIdx.x * 256 + threadIdx.x] = acc;   // keeps the MFMAs alive
+}
+
 }  // namespace
+
+hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, hipStream_t s) {
+  hipLaunchKernelGGL(calib_mfma_kernel, dim3(workgroups), dim3(256), 0, s, sink, iters);
+  return hipGetLastError();
+}
 
 hipError_t launch_calib_copy(void* dst, const void* src, size_t bytes, hipStream_t s) {
   const size_t n16 = bytes / 16;

@@ -105,5 +105,6 @@ hipError_t launch_kv_gather(const void* src, uint32_t src_dtype, void* dst, uint
                             uint32_t ring_mask, hipStream_t s);
 
 hipError_t launch_calib_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
+hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, hipStream_t s);
 
 }  // namespace dg

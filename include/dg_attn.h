@@ -173,6 +173,14 @@ int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches);
  * profiler counters are scaled by.  Measurement aid, no counterpart in the reference. */
 int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream);
 
+/* Launch of nothing but bf16 32x32x16 MFMAs (`workgroups` x 4 waves x `iters` x 16) writing
+ * `*flops` = the floating-point operations it performs; the caller times it.  `sink` (at
+ * least workgroups*256 floats, device memory) is never written in practice.  What this
+ * sustains is the MFMA ceiling of the machine at hand, next to which the attention kernel's
+ * rate is read.  Measurement aid, no counterpart in the reference. */
+int dg_calib_mfma(float* sink, size_t sink_bytes, uint32_t workgroups, uint32_t iters, uint64_t* flops,
+                  void* stream);
+
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);
 uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slots, uint32_t kv_dtype);
