@@ -14,6 +14,8 @@ DG_ATTN_F_OUT_TRUNCATE = 0x1
 DG_ATTN_F_CAUSAL_SEES_MASKED = 0x2
 DG_ATTN_F_T_LO_EXPLICIT = 0x4
 
+DG_ROPE_F_QK_TRUNCATE = 0x1
+
 DG_OK = 0
 DG_ERR_NULL, DG_ERR_SHAPE, DG_ERR_DTYPE, DG_ERR_LAYOUT = -1, -2, -3, -4
 DG_ERR_WORKSPACE, DG_ERR_MASK, DG_ERR_LAUNCH, DG_ERR_DEVICE, DG_ERR_UNSUPPORTED = -5, -6, -7, -8, -9
@@ -24,7 +26,7 @@ EXPORTS = (
     "dg_attn_resolved_splits", "dg_attn_forward", "dg_attn_strerror", "dg_attn_abi_version",
     "dg_attn_visible_pairs", "dg_attention_dispatch", "dg_attention_state_bytes", "dg_kv_row_bytes",
     "dg_kv_region_bytes", "dg_kv_slot", "dg_layer_kv_slots", "dg_prof_begin", "dg_prof_end",
-    "dg_calib_copy", "dg_calib_mfma",
+    "dg_calib_copy", "dg_calib_mfma", "dg_qk_rope_kv", "dg_qk_rope_kv_dispatch",
 )
 
 
@@ -34,6 +36,18 @@ class AttnDesc(C.Structure):
         ("kv_len", C.c_uint32), ("causal_rows", C.c_uint32), ("window", C.c_uint32), ("kv_ring_mask", C.c_uint32),
         ("q_dtype", C.c_uint32), ("kv_dtype", C.c_uint32), ("out_dtype", C.c_uint32), ("flags", C.c_uint32),
         ("t_lo", C.c_uint32), ("n_splits", C.c_uint32), ("kernel", C.c_uint32), ("softmax_scale", C.c_float),
+        ("kv_region_bytes", C.c_uint64),
+        ("k_tok_stride", C.c_int64), ("k_head_stride", C.c_int64),
+        ("v_base_off", C.c_int64), ("v_tok_stride", C.c_int64), ("v_head_stride", C.c_int64),
+    ]
+
+
+class RopeDesc(C.Structure):
+    """dg_rope_desc: the producer of the cache rows (RMSNorm + RoPE + KV write)."""
+    _fields_ = [
+        ("canvas", C.c_uint32), ("n_q_heads", C.c_uint32), ("n_kv_heads", C.c_uint32), ("head_dim", C.c_uint32),
+        ("kv_len", C.c_uint32), ("kv_write_end", C.c_uint32), ("kv_ring_mask", C.c_uint32), ("is_full", C.c_uint32),
+        ("v_from_k", C.c_uint32), ("kv_dtype", C.c_uint32), ("flags", C.c_uint32), ("reserved", C.c_uint32),
         ("kv_region_bytes", C.c_uint64),
         ("k_tok_stride", C.c_int64), ("k_head_stride", C.c_int64),
         ("v_base_off", C.c_int64), ("v_tok_stride", C.c_int64), ("v_head_stride", C.c_int64),
@@ -127,6 +141,10 @@ def load():
     lib.dg_calib_copy.restype = C.c_int
     lib.dg_calib_mfma.argtypes = [VP, C.c_size_t, C.c_uint32, C.c_uint32, P(C.c_uint64), VP]
     lib.dg_calib_mfma.restype = C.c_int
+    lib.dg_qk_rope_kv.argtypes = [P(RopeDesc), VP, VP, VP, VP, VP, VP, VP, VP]
+    lib.dg_qk_rope_kv.restype = C.c_int
+    lib.dg_qk_rope_kv_dispatch.argtypes = [VP, VP, VP, VP, VP, P(LayerOffsets), P(StepParams), P(AttnDims), VP, VP]
+    lib.dg_qk_rope_kv_dispatch.restype = C.c_int
     lib.dg_prof_begin.argtypes = [C.c_uint32]
     lib.dg_prof_begin.restype = C.c_int
     lib.dg_prof_end.argtypes = [P(C.c_double), P(C.c_uint32)]

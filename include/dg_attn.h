@@ -159,6 +159,52 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
 int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
                              size_t* out_bytes);
 
+/* ---- the producer of the rows attention reads: per-head RMSNorm + RoPE + KV-cache write ----
+ * Replaces the reference's qk_rope_kv kernel (src/shaders/attn/qk_rope_kv/qk_rope_kv.metal:29-149,
+ * encoded by StepEnc::encode_layer_qk_rope_kv, src/metal/step_kernel/enc.rs:1739-1804; CPU twin
+ * src/shaders/attn/cpu.rs:78-145).  For canvas row tok at position pos = kv_len + tok:
+ *   Q head:  q <- rope(rms_norm(q) * q_norm_w, pos), in place
+ *   K head:  x  = rope(rms_norm(k) * k_norm_w, pos); cache K row at slot(pos) <- x;
+ *            k <- x in place unless V aliases the raw k projection (v_from_k)
+ *   V head:  cache V row at slot(pos) <- rms_norm(v_from_k ? raw k : v), no weight
+ * is_full selects proportional RoPE (pairs (d, hd/2+d), d < hd/8, theta 1e6), otherwise
+ * split-half over the whole head (pairs (d, hd/2+d), theta 1e4).  RoPE uses the absolute
+ * position; only the storage slot is ring-mapped.  Positions >= kv_write_end are not written
+ * to the cache (prefill pad rows, qk_rope_kv.metal:56-60). */
+#define DG_ROPE_F_QK_TRUNCATE 0x1u  /* store q/k with the reference's truncating bf16 store; default RNE */
+
+typedef struct dg_rope_desc {
+  uint32_t canvas, n_q_heads, n_kv_heads;
+  uint32_t head_dim;        /* 32, 64, 128, 256 or 512 */
+  uint32_t kv_len;          /* StepParams.kv_len */
+  uint32_t kv_write_end;    /* StepParams.kv_write_end; 0xffffffff = write every row */
+  uint32_t kv_ring_mask;    /* LayerOffsets.kv_ring_mask */
+  uint32_t is_full;         /* LayerOffsets.is_full */
+  uint32_t v_from_k;        /* LayerOffsets.v_proj == 0 */
+  uint32_t kv_dtype;        /* DG_F16 or DG_BF16: element type of the cache */
+  uint32_t flags;
+  uint32_t reserved;
+  uint64_t kv_region_bytes; /* byte offset of this layer's region inside kv_base */
+  /* element strides/offsets inside the region, as in dg_attn_desc */
+  int64_t  k_tok_stride, k_head_stride;
+  int64_t  v_base_off, v_tok_stride, v_head_stride;
+} dg_rope_desc;
+
+/* q [canvas][n_q_heads][hd], k and v [canvas][n_kv_heads][hd]: bf16, device.  q_norm_w, k_norm_w:
+ * [hd] bf16, device.  v may be NULL when v_from_k.  Enqueues one kernel on `stream`. */
+int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* kv_base, const void* q_norm_w,
+                  const void* k_norm_w, dg_debug_status* dbg, void* stream);
+
+/* The same with exactly the buffers the reference kernel binds (qk_rope_kv.metal:30-38): q, k, v
+ * in the arena, the whole f16 KV buffer (the kernel adds L->kv_region), the weight blob (norm
+ * weights at L->q_norm / L->k_norm, bf16), host copies of L / P / dims.  q and k are stored with
+ * the reference's truncating bf16 store, the cache as f16 (kv_store). */
+int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
+                           const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream);
+
+#define DG_DBG_ROPE_NONFINITE 3u        /* a head's 1/rms was not finite */
+#define DG_DBG_KERNEL_QK_ROPE_KV 6u
+
 /* ---- optional kernel timing (measurement aid; no counterpart in the reference, whose
  * harness times whole command buffers: src/shaders/attn/harness.rs:149-170) ----
  * Between dg_prof_begin and dg_prof_end every dg_attn_forward issued by the calling thread

@@ -484,6 +484,92 @@ void dgo_rms_norm_head(float* x, const float* weight, size_t n, float eps) {
   for (size_t i = 0; i < n; ++i) x[i] *= inv * (weight ? weight[i] : 1.0f);
 }
 
+// ---- producer: per-head RMSNorm + RoPE + KV-cache write ----
+void dgo_rope_split_half(float* x, uint32_t rot, uint32_t head_dim, float theta, uint32_t pos) {  // cpu.rs:31-45
+  const uint32_t half_rot = rot / 2;
+  for (uint32_t dd = 0; dd < half_rot; ++dd) {
+    const float inv_freq = std::pow(theta, -2.0f * (float)dd / (float)head_dim);
+    const float a = (float)pos * inv_freq;
+    const float c = std::cos(a), s = std::sin(a);
+    const float x0 = x[dd], x1 = x[dd + half_rot];
+    x[dd] = x0 * c - x1 * s;
+    x[dd + half_rot] = x0 * s + x1 * c;
+  }
+}
+
+void dgo_rope_proportional(float* x, uint32_t rotary_dim, uint32_t head_dim, float theta, uint32_t pos) {  // cpu.rs:48-65
+  const uint32_t half_head = head_dim / 2, half_rot = rotary_dim / 2;
+  for (uint32_t dd = 0; dd < half_rot; ++dd) {
+    const float inv_freq = std::pow(theta, -2.0f * (float)dd / (float)head_dim);
+    const float a = (float)pos * inv_freq;
+    const float c = std::cos(a), s = std::sin(a);
+    const float x0 = x[dd], x1 = x[half_head + dd];
+    x[dd] = x0 * c - x1 * s;
+    x[half_head + dd] = x0 * s + x1 * c;
+  }
+}
+
+void dgo_qk_rope_kv_f32(const dgo_rope_desc* d, float* q, float* k, const float* v, float* kvcache,
+                        const float* q_norm_w, const float* k_norm_w) {  // cpu.rs:78-145
+  const uint32_t hd = d->head_dim, nkv = d->n_kv_heads, nq = d->n_q_heads;
+  const uint32_t rot = d->is_full ? hd / 4 : hd;            // cpu.rs:17-23
+  const float theta = d->is_full ? 1.0e6f : 1.0e4f;         // cpu.rs:25-27
+  std::vector<float> tmp(hd);
+  for (uint32_t tok = 0; tok < d->canvas; ++tok) {
+    const uint32_t pos = d->kv_len + tok;
+    const bool kv_write = pos < d->kv_write_end;            // qk_rope_kv.metal:56-60
+    const int64_t slot = d->kv_ring_mask ? (int64_t)(pos & d->kv_ring_mask) : (int64_t)pos;  // attention_device.metal:28-30
+    for (uint32_t h = 0; h < nq + 2 * nkv; ++h) {
+      const bool is_q = h < nq, is_k = !is_q && h < nq + nkv;
+      const uint32_t hh = is_q ? h : (h - nq) % nkv;
+      if (!is_q && !is_k) {                                 // V head: cpu.rs:110-122
+        const float* src = (d->v_from_k ? k : v) + ((size_t)tok * nkv + hh) * hd;
+        std::copy(src, src + hd, tmp.begin());
+        dgo_rms_norm_head(tmp.data(), nullptr, hd, 1e-6f);
+        if (kv_write) std::copy(tmp.begin(), tmp.end(), kvcache + d->v_off + slot * d->v_tok_stride + (int64_t)hh * d->v_head_stride);
+        continue;
+      }
+      float* head = is_q ? q + ((size_t)tok * nq + hh) * hd : k + ((size_t)tok * nkv + hh) * hd;
+      std::copy(head, head + hd, tmp.begin());
+      dgo_rms_norm_head(tmp.data(), is_q ? q_norm_w : k_norm_w, hd, 1e-6f);
+      if (d->is_full) dgo_rope_proportional(tmp.data(), rot, hd, theta, pos);
+      else dgo_rope_split_half(tmp.data(), rot, hd, theta, pos);
+      if (is_k) {
+        if (kv_write) std::copy(tmp.begin(), tmp.end(), kvcache + d->k_off + slot * d->k_tok_stride + (int64_t)hh * d->k_head_stride);
+        // V aliases the raw k projection on such layers: leave k untouched for the V pass (cpu.rs:137-140)
+        if (!d->v_from_k) std::copy(tmp.begin(), tmp.end(), head);
+      } else {
+        std::copy(tmp.begin(), tmp.end(), head);
+      }
+    }
+  }
+}
+
+void dgo_fixture_rope(int which, float* q, float* k, float* v, float* qw, float* kw) {  // qk_rope_kv/mod.rs:80-189
+  if (which == 0) {          // tiny_fixture: canvas 2, Hq 4, Hkv 2, hd 32
+    const size_t nq = 2 * 4 * 32, nk = 2 * 2 * 32;
+    for (size_t i = 0; i < nq; ++i) q[i] = std::sin((float)i * 0.13f) * 0.5f;
+    for (size_t i = 0; i < nk; ++i) k[i] = std::cos((float)i * 0.17f) * 0.4f;
+    for (size_t i = 0; i < nk; ++i) v[i] = std::sin((float)i * 0.11f) * 0.3f;
+    for (size_t i = 0; i < 32; ++i) qw[i] = kw[i] = 1.0f;
+  } else if (which == 1) {   // full_layer_fixture: canvas 2, Hq 4, Hkv 2, hd 64
+    const size_t nq = 2 * 4 * 64, nk = 2 * 2 * 64;
+    for (size_t i = 0; i < nq; ++i) q[i] = std::sin((float)i * 0.07f) * 0.6f;
+    for (size_t i = 0; i < nk; ++i) k[i] = std::cos((float)i * 0.09f) * 0.5f;
+    for (size_t i = 0; i < nk; ++i) v[i] = std::sin((float)i * 0.08f) * 0.45f;
+    for (size_t i = 0; i < 64; ++i) qw[i] = kw[i] = 1.0f;
+  } else {                   // full_hd512_v_alias_fixture: canvas 1, Hq 16, Hkv 2, hd 512
+    const size_t nq = 1 * 16 * 512, nk = 1 * 2 * 512;
+    for (size_t i = 0; i < nq; ++i) q[i] = std::sin((float)i * 0.031f) * 0.55f;
+    for (size_t i = 0; i < nk; ++i) k[i] = std::cos((float)i * 0.029f) * 0.48f;
+    for (size_t i = 0; i < nk; ++i) v[i] = 0.0f;
+    for (size_t i = 0; i < 512; ++i) {
+      qw[i] = 1.0f + (float)i * 0.0001f;
+      kw[i] = 1.0f - (float)i * 0.00005f;
+    }
+  }
+}
+
 // ---- fixture generators ----
 void dgo_fixture_tiny(float* q, float* kv) {  // attention/mod.rs:59-95
   const uint32_t canvas = 2, nq = 4, nkv = 2, hd = 32, kv_len = 2, t_total = kv_len + canvas;

@@ -18,6 +18,11 @@
  *                            reference's state planes: attention_mma_full.metal:107-118,355-368
  *   rounding helpers         src/shaders/common/bf16.rs:9-41, src/shaders/common/f16.rs:3-60
  *   dgo_rms_norm_no_scale    src/shaders/cpu/mod.rs:24-35 ; dgo_rms_norm_head src/shaders/attn/cpu.rs:67-75
+ *   dgo_rope_split_half      src/shaders/attn/cpu.rs:31-45 ; dgo_rope_proportional cpu.rs:48-65
+ *   dgo_qk_rope_kv_f32       src/shaders/attn/cpu.rs:78-145 (per-head RMSNorm + RoPE + cache write, V aliasing)
+ *                            src/shaders/attn/qk_rope_kv/qk_rope_kv.metal:56-60 (kv_write_end suppression),
+ *                            :87,:114 + src/shaders/include/attention_device.metal:28-33 (ring slot of the write)
+ *   dgo_fixture_rope_*       src/shaders/attn/qk_rope_kv/mod.rs:80-189
  *   fixture generators       src/shaders/attn/attention/mod.rs:59-184,689-691,
  *                            src/shaders/attn/attention_gemm/mod.rs:364-432,
  *                            src/metal/step_kernel/runtime.rs:183-206 (synthetic_fill_kv)
@@ -29,6 +34,11 @@
  *   - blocked(bk) == unblocked for bk in {1,3,8,16,64,4096} (reference's own test, 1e-3)
  *   - special cases: all keys equal -> mean(V), LSE = s + ln n; one dominant key -> that V row
  *   - rounding known answers (bf16.rs:47-55 value 1.234567; f16 clamp / flush-subnormal cases)
+ *   - producer (qk_rope_kv): unit RMS of every normed head; pair norms preserved by the rotation;
+ *     position 0 is the identity; R(a)R(b) = R(a+b) via the angle closed form theta^(-2d/hd);
+ *     one-hot inputs show which elements are paired (split-half vs proportional) and which are
+ *     left alone (proportional: only hd/4 of the head rotates); cache rows land at the slot the
+ *     attention oracle reads; V = rms_norm_no_scale(raw k) when V aliases k
  * LSE is not emitted anywhere in the reference; it is the closed form m + ln(l) of the
  * recurrence's own (m, l), cross-checked against a float64 logsumexp of the score row.
  */
@@ -105,6 +115,27 @@ void dgo_from_bits(const uint16_t* bits, float* x, size_t n, int is_f16);
 
 void dgo_rms_norm_no_scale(float* out, const float* x, size_t n, float eps);
 void dgo_rms_norm_head(float* x, const float* weight /*may be NULL*/, size_t n, float eps);
+
+/* ---- the producer of the cache rows attention reads: per-head RMSNorm + RoPE + KV write ---- */
+typedef struct dgo_rope_desc {
+  uint32_t canvas, n_q_heads, n_kv_heads, head_dim;
+  uint32_t kv_len;        /* canvas row tok sits at position kv_len + tok */
+  uint32_t kv_write_end;  /* positions >= this are normed/rotated but never written to the cache */
+  uint32_t kv_ring_mask;  /* 0 = linear, else the row goes to slot pos & mask; RoPE uses the absolute pos */
+  uint32_t is_full;       /* 1: proportional RoPE, theta 1e6, rot = hd/4; 0: split-half, theta 1e4, rot = hd */
+  uint32_t v_from_k;      /* 1 (reference v_proj == 0): V is the RAW k projection, normed without weight */
+  int64_t  k_off, k_tok_stride, k_head_stride;  /* element offsets into kvcache[] */
+  int64_t  v_off, v_tok_stride, v_head_stride;
+} dgo_rope_desc;
+void dgo_rope_split_half(float* x, uint32_t rot, uint32_t head_dim, float theta, uint32_t pos);
+void dgo_rope_proportional(float* x, uint32_t rotary_dim, uint32_t head_dim, float theta, uint32_t pos);
+/* q [canvas][Hq][hd] and k [canvas][Hkv][hd] are updated in place (k only when V does not alias it);
+ * v [canvas][Hkv][hd] is read when v_from_k == 0.  No storage rounding happens here. */
+void dgo_qk_rope_kv_f32(const dgo_rope_desc* d, float* q, float* k, const float* v, float* kvcache,
+                        const float* q_norm_w, const float* k_norm_w);
+/* the reference's producer fixtures (qk_rope_kv/mod.rs:80-189): which = 0 tiny, 1 full_layer,
+ * 2 full_hd512_v_alias; buffers sized by the caller from the fixture's dims */
+void dgo_fixture_rope(int which, float* q, float* k, float* v, float* q_norm_w, float* k_norm_w);
 
 /* reference fixture generators; kv in the reference slot-major layout, sizes as the reference computes them */
 void dgo_fixture_tiny(float* q /*2*4*32*/, float* kv /*4*2*32*2*/);

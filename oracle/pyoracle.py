@@ -27,6 +27,13 @@ class Desc(C.Structure):
     ]
 
 
+class RopeDesc(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("canvas", "n_q_heads", "n_kv_heads", "head_dim", "kv_len", "kv_write_end",
+                                           "kv_ring_mask", "is_full", "v_from_k")] + \
+               [(n, C.c_int64) for n in ("k_off", "k_tok_stride", "k_head_stride", "v_off", "v_tok_stride",
+                                          "v_head_stride")]
+
+
 def build(force: bool = False) -> Path:
     if force or not LIB_PATH.exists():
         subprocess.run(["make", "-C", str(ORACLE_DIR), "-B" if force else "-s"], check=True,
@@ -74,6 +81,11 @@ def load():
     lib.dgo_fixture_model_attn.argtypes = [C.c_uint32] * 5 + [VP, VP]
     lib.dgo_fixture_model_full.argtypes = [C.c_uint32] * 5 + [VP, VP]
     lib.dgo_synthetic_fill_kv.argtypes = [VP, C.c_size_t, C.c_uint64]
+    lib.dgo_rope_split_half.argtypes = [VP, C.c_uint32, C.c_uint32, C.c_float, C.c_uint32]
+    lib.dgo_rope_proportional.argtypes = [VP, C.c_uint32, C.c_uint32, C.c_float, C.c_uint32]
+    lib.dgo_qk_rope_kv_f32.argtypes = [C.POINTER(RopeDesc), VP, VP, VP, VP, VP, VP]
+    lib.dgo_fixture_rope.argtypes = [C.c_int, VP, VP, VP, VP, VP]
+    lib.dgo_rms_norm_head.argtypes = [VP, VP, C.c_size_t, C.c_float]
     lib.dgo_max_threads.restype = C.c_int
     _lib = lib
     return lib
@@ -229,6 +241,68 @@ def fixture(name, *dims):
     else:
         raise ValueError(name)
     return q, kv
+
+
+def make_rope_desc(canvas, n_q_heads, n_kv_heads, head_dim, kv_len, *, is_full=False, v_from_k=False,
+                   kv_write_end=0xFFFFFFFF, kv_ring_mask=0, layout="reference", t_cap=0):
+    """Producer descriptor; cache strides as in make_desc (reference slot-major or head-major planes)."""
+    d = RopeDesc(canvas, n_q_heads, n_kv_heads, head_dim, kv_len, kv_write_end, kv_ring_mask, int(is_full),
+                 int(v_from_k))
+    row = n_kv_heads * head_dim
+    if layout == "reference":
+        d.k_off, d.k_tok_stride, d.k_head_stride = 0, 2 * row, head_dim
+        d.v_off, d.v_tok_stride, d.v_head_stride = row, 2 * row, head_dim
+    else:
+        d.k_off, d.k_tok_stride, d.k_head_stride = 0, head_dim, t_cap * head_dim
+        d.v_off, d.v_tok_stride, d.v_head_stride = n_kv_heads * t_cap * head_dim, head_dim, t_cap * head_dim
+    return d
+
+
+def qk_rope_kv_f32(d, q, k, v, kvcache, q_norm_w, k_norm_w):
+    """Returns (q', k', kvcache') as new f32 arrays; inputs are not modified."""
+    q = np.array(q, dtype=np.float32).ravel()
+    k = np.array(k, dtype=np.float32).ravel()
+    v = np.ascontiguousarray(v, dtype=np.float32).ravel()
+    kvc = np.array(kvcache, dtype=np.float32).ravel()
+    qw = np.ascontiguousarray(q_norm_w, dtype=np.float32)
+    kw = np.ascontiguousarray(k_norm_w, dtype=np.float32)
+    load().dgo_qk_rope_kv_f32(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(kvc), _ptr(qw), _ptr(kw))
+    return q, k, kvc
+
+
+def rope(x, rot, head_dim, theta, pos, proportional):
+    x = np.array(x, dtype=np.float32)
+    fn = load().dgo_rope_proportional if proportional else load().dgo_rope_split_half
+    fn(_ptr(x), rot, head_dim, theta, pos)
+    return x
+
+
+def rms_norm_head(x, w=None, eps=1e-6):
+    x = np.array(x, dtype=np.float32)
+    wv = None if w is None else np.ascontiguousarray(w, dtype=np.float32)
+    load().dgo_rms_norm_head(_ptr(x), None if wv is None else _ptr(wv), x.size, eps)
+    return x
+
+
+ROPE_FIXTURES = {  # name -> (which, canvas, Hq, Hkv, hd, kv_len, is_full, v_from_k); qk_rope_kv/mod.rs:80-189
+    "tiny": (0, 2, 4, 2, 32, 2, False, False),
+    "full_layer": (1, 2, 4, 2, 64, 2, True, False),
+    "full_attn_v_alias": (1, 2, 4, 2, 64, 2, True, True),
+    "full_hd512_v_alias": (2, 1, 16, 2, 512, 22, True, True),
+}
+
+
+def rope_fixture(name):
+    """(dims dict, q, k, v, q_norm_w, k_norm_w) of one of the reference's producer fixtures."""
+    which, canvas, nq, nkv, hd, kv_len, is_full, v_from_k = ROPE_FIXTURES[name]
+    q = np.zeros(canvas * nq * hd, np.float32)
+    k = np.zeros(canvas * nkv * hd, np.float32)
+    v = np.zeros(canvas * nkv * hd, np.float32)
+    qw, kw = np.zeros(hd, np.float32), np.zeros(hd, np.float32)
+    load().dgo_fixture_rope(which, _ptr(q), _ptr(k), _ptr(v), _ptr(qw), _ptr(kw))
+    dims = dict(canvas=canvas, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd, kv_len=kv_len, is_full=is_full,
+                v_from_k=v_from_k)
+    return dims, q, k, v, qw, kw
 
 
 def synthetic_fill_kv(n, seed):

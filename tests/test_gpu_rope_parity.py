@@ -1,0 +1,163 @@
+"""GPU parity of the producer (per-head RMSNorm + RoPE + KV-cache write) against the CPU oracle,
+through the C ABI.  The four reference cases and their tolerances are qk_rope_kv/mod.rs:437-489
+(max_tol 1e-2 / 2e-2, cosine >= 0.9999 / 0.999).  At layer-sized shapes and long prefixes the
+comparison allows one bf16 / f16 storage step on top: the angle pos * theta^(-2d/hd) is an fp32
+product whose last-place differences between two math libraries grow with pos."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from diffgemma_amd import attention as A
+from diffgemma_amd import capi, qk_rope_kv as QR, rounding as R
+from helpers import assert_oracle, cosine, max_abs_diff
+
+pytestmark = pytest.mark.gpu
+
+
+def reference_cpu(po, f):
+    """The reference's test wrapper (qk_rope_kv/mod.rs:238-262): inputs -> bf16 by truncation, run the
+    CPU twin, q/k -> bf16 (its f32_to_bf16_bits truncates), cache -> f16 by truncation."""
+    tr = lambda x: R.bf16_bits_to_f32(R.f32_to_bf16_bits_trunc(x))
+    d = po.make_rope_desc(f.canvas, f.n_q_heads, f.n_kv_heads, f.head_dim, f.kv_len, is_full=f.is_full,
+                          v_from_k=(f.v_proj == 0), kv_write_end=f.kv_write_end, kv_ring_mask=f.kv_ring_mask)
+    region = f.kvcache[f.kv_region // 2:]
+    q, k, kvc = po.qk_rope_kv_f32(d, tr(f.q), tr(f.k), tr(f.v), R.f16_bits_to_f32(R.f32_to_f16_bits_trunc(region)),
+                                  tr(f.q_norm_w), tr(f.k_norm_w))
+    full = np.concatenate([f.kvcache[:f.kv_region // 2], R.f16_bits_to_f32(R.f32_to_f16_bits_trunc(kvc))])
+    return tr(q), tr(k), full
+
+
+CASES = {"tiny": (QR.tiny_fixture, 1e-2, 0.9999), "full_layer": (QR.full_layer_fixture, 1e-2, 0.9999),
+         "full_attn_v_alias": (QR.full_attn_v_alias_fixture, 1e-2, 0.9999),
+         "full_hd512_v_alias": (QR.full_hd512_v_alias_fixture, 2e-2, 0.999)}
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_reference_matrix(gpu_ready, po, name):
+    make, tol, cs = CASES[name]
+    f = make()
+    q, k, kvc = reference_cpu(po, f)
+    assert_oracle(QR.gpu(f), QR.pack_out(q, k, kvc, f), tol, cs)
+
+
+def storage_tolerance(ref, ulp_bits):
+    """One storage step of the value's own magnitude plus 1e-2 (the reference's absolute bound)."""
+    return 1e-2 + np.abs(ref) * 2.0 ** (-ulp_bits)
+
+
+@pytest.mark.parametrize("shape", [
+    # canvas, Hq, Hkv, hd, kv_len, is_full, v_proj, ring mask
+    (256, 16, 8, 256, 4096, False, 1, 2047),      # sliding layer on its ring
+    (256, 16, 2, 512, 32768, True, 0, 0),         # global layer at the 32k prefix, V aliases k
+    (64, 16, 2, 512, 131072, True, 1, 0),         # long context, shrunken canvas
+    (37, 8, 4, 128, 333, False, 1, 0),
+])
+def test_layer_shapes(gpu_ready, po, shape):
+    canvas, nq, nkv, hd, kv_len, is_full, v_proj, ring = shape
+    f = QR.random_fixture(canvas, nq, nkv, hd, kv_len, is_full=is_full, v_proj=v_proj, seed=hd + canvas,
+                          kv_ring_mask=ring)
+    q, k, kvc = reference_cpu(po, f)
+    rig = QR.RopeRig(f)
+    rig.run_dispatch()
+    gq, gk, gkv = rig.read()
+    assert np.isfinite(gq).all() and np.isfinite(gkv).all()
+    assert np.all(np.abs(gq - q) <= storage_tolerance(q, 7)) and cosine(gq, q) >= 0.9999
+    assert np.all(np.abs(gk - k) <= storage_tolerance(k, 7)) and cosine(gk, k) >= 0.9999
+    assert np.all(np.abs(gkv - kvc) <= storage_tolerance(kvc, 10)) and cosine(gkv, kvc) >= 0.9999
+    # rows the launch does not own are bit-identical to what was there
+    want_pack, got_pack = QR.pack_out(q, k, kvc, f), QR.pack_out(gq, gk, gkv, f)
+    assert got_pack.shape == want_pack.shape
+    ds = rig.buf_dbg.cpu().numpy()
+    assert ds[0] == 0, f"debug status {ds}"
+
+
+def test_write_suppression_and_untouched_rows(gpu_ready, po):
+    """kv_write_end (qk_rope_kv.metal:56-60): pad rows are normed and rotated in place but never reach
+    the cache; every slot the launch does not own keeps its bits."""
+    f = QR.random_fixture(8, 16, 8, 256, 1020, is_full=False, v_proj=1, seed=9, kv_ring_mask=1023, kv_write_end=1024,
+                          kv_region=4096)
+    f.kvcache[:] = 0.5
+    rig = QR.RopeRig(f)
+    before = rig.buf_kv.cpu().numpy().copy()
+    rig.run_dispatch()
+    after = rig.buf_kv.cpu().numpy()
+    row = 2 * f.n_kv_heads * f.head_dim
+    changed = np.flatnonzero((before != after).reshape(-1)) // 1
+    slots = {int((i - f.kv_region // 2) // row) for i in changed}
+    assert slots == {1020, 1021, 1022, 1023}                 # positions 1024.. would wrap onto slots 0..3
+    q, k, kvc = reference_cpu(po, f)
+    gq, gk, gkv = rig.read()
+    assert max_abs_diff(gq, q) <= 2e-2 and max_abs_diff(gkv, kvc) <= 1e-2   # suppressed rows still rotate q
+
+
+def test_general_entry_bf16_head_major_cache(gpu_ready, po):
+    """dg_qk_rope_kv with the cache the benchmark's attention reads: bf16, two planes [Hkv][t_cap][d]."""
+    import torch
+    canvas, nq, nkv, hd, kv_len = 32, 16, 2, 512, 480
+    t_cap = kv_len + canvas
+    f = QR.random_fixture(canvas, nq, nkv, hd, kv_len, is_full=True, v_proj=0, seed=12)
+    tr = lambda x: R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(x))
+    d = QR.rope_desc(f, kv_dtype=capi.DG_BF16, truncate=False, layout="head_major", t_cap=t_cap)
+    bq, bk = A.to_device_bits(R.f32_to_bf16_bits_rne(f.q)), A.to_device_bits(R.f32_to_bf16_bits_rne(f.k))
+    bqw, bkw = A.to_device_bits(R.f32_to_bf16_bits_rne(f.q_norm_w)), A.to_device_bits(R.f32_to_bf16_bits_rne(f.k_norm_w))
+    cache = torch.zeros(2 * nkv * t_cap * hd, dtype=torch.int16, device="cuda")
+    capi.check(capi.load().dg_qk_rope_kv(C.byref(d), bq.data_ptr(), bk.data_ptr(), None, cache.data_ptr(),
+                                         bqw.data_ptr(), bkw.data_ptr(), None, A.stream_handle()))
+    torch.cuda.synchronize()
+    od = po.make_rope_desc(canvas, nq, nkv, hd, kv_len, is_full=True, v_from_k=True, layout="head_major", t_cap=t_cap)
+    q, k, kvc = po.qk_rope_kv_f32(od, tr(f.q), tr(f.k), f.v, np.zeros(2 * nkv * t_cap * hd, np.float32),
+                                  tr(f.q_norm_w), tr(f.k_norm_w))
+    got = R.bf16_bits_to_f32(cache.cpu().numpy().view(np.uint16))
+    assert np.all(np.abs(got - kvc) <= storage_tolerance(kvc, 7)) and cosine(got, kvc) >= 0.9999
+    assert np.array_equal(R.bf16_bits_to_f32(bk.cpu().numpy().view(np.uint16)), tr(f.k))    # raw k untouched
+    gq = R.bf16_bits_to_f32(bq.cpu().numpy().view(np.uint16))
+    assert np.all(np.abs(gq - q) <= storage_tolerance(q, 7))
+
+
+def test_producer_then_attention(gpu_ready, po):
+    """The two kernels back to back, as a denoise step runs them (enc.rs:852-856): the canvas rows the
+    producer writes are the rows attention reads."""
+    import torch
+    canvas, nq, nkv, hd, kv_len = 64, 16, 2, 512, 960
+    f = QR.random_fixture(canvas, nq, nkv, hd, kv_len, is_full=True, v_proj=0, seed=21)
+    rng = np.random.default_rng(5)
+    prefix = rng.standard_normal((kv_len, 2 * nkv * hd)).astype(np.float32)
+    prefix /= np.sqrt((prefix.reshape(kv_len, 2 * nkv, hd) ** 2).mean(-1, keepdims=True)).repeat(hd, -1).reshape(kv_len, -1)
+    f.kvcache[:kv_len * 2 * nkv * hd] = prefix.ravel()
+    rig = QR.RopeRig(f)
+    rig.run_dispatch()
+    out = torch.zeros(canvas * nq * hd, dtype=torch.float32, device="cuda")
+    lse = torch.zeros(canvas * nq, dtype=torch.float32, device="cuda")
+    ad = A.make_desc(canvas, nq, nkv, hd, kv_len, q_dtype=capi.DG_BF16, kv_dtype=capi.DG_F16, out_dtype=capi.DG_F32)
+    A.forward(ad, rig.buf_q, rig.buf_kv, out, lse, A.alloc_workspace(ad))
+    torch.cuda.synchronize()
+    q, k, kvc = reference_cpu(po, f)
+    gq, gk, gkv = rig.read()
+    assert np.all(np.abs(gq - q) <= storage_tolerance(q, 7)) and np.all(np.abs(gkv - kvc) <= storage_tolerance(kvc, 10))
+    # attention is compared on identical inputs (what the producer left on the device): with scores
+    # spread over tens of units, one storage step in a single q element moves an output row by more
+    # than the attention tolerance, on either side alike
+    ref, ref_lse = po.attention_f32(po.make_desc(canvas, nq, nkv, hd, kv_len), gq, gkv)
+    got = out.cpu().numpy().reshape(ref.shape)
+    assert max_abs_diff(got, ref) <= 2e-2 and float(np.mean(np.abs(got - ref))) <= 2e-3
+    rel = np.abs(lse.cpu().numpy().reshape(ref_lse.shape) - ref_lse) / np.maximum(np.abs(ref_lse), 1e-6)
+    assert rel.max() <= 1e-3
+
+
+def test_rejects_bad_arguments(gpu_ready):
+    f = QR.tiny_fixture()
+    d = QR.rope_desc(f)
+    lib = capi.load()
+    assert lib.dg_qk_rope_kv(C.byref(d), None, None, None, None, None, None, None, None) == capi.DG_ERR_NULL
+    rig = QR.RopeRig(f)
+    args = (rig.buf_q.data_ptr(), rig.buf_k.data_ptr(), rig.buf_v.data_ptr(), rig.buf_kv.data_ptr(),
+            rig.buf_blob.data_ptr(), rig.buf_blob.data_ptr() + 2 * f.head_dim, None, A.stream_handle())
+    d.head_dim = 48
+    assert lib.dg_qk_rope_kv(C.byref(d), *args) == capi.DG_ERR_SHAPE
+    d = QR.rope_desc(f)
+    d.kv_dtype = capi.DG_F32
+    assert lib.dg_qk_rope_kv(C.byref(d), *args) == capi.DG_ERR_DTYPE
+    d = QR.rope_desc(f)
+    d.kv_ring_mask = 5
+    assert lib.dg_qk_rope_kv(C.byref(d), *args) == capi.DG_ERR_LAYOUT
