@@ -69,6 +69,76 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
 MEASURED_HBM_BYTES_PER_LAUNCH = {"cfg3_global": 169.8e6 + 72.4e6}
 
 
+PRODUCER_SHAPES = {   # canvas, Hq, Hkv, hd, kv_len, is_full, v_proj, ring mask: the two layer types of the 30-layer stack
+    "qk_rope_kv_global": (256, 16, 2, 512, 32768, True, 0, 0),
+    "qk_rope_kv_sliding": (256, 16, 8, 256, 32768, False, 1, 2047),
+}
+
+
+def bench_producer(args):
+    """One step = one dg_qk_rope_kv launch (per-head RMSNorm + RoPE + KV-cache write) for one layer."""
+    import torch
+    from diffgemma_amd import attention as A, capi, qk_rope_kv as QR, rounding as R
+    from oracle import pyoracle as po
+    canvas, nq, nkv, hd, kv_len, is_full, v_proj, ring = PRODUCER_SHAPES[args.workload]
+    f = QR.random_fixture(canvas, nq, nkv, hd, kv_len, is_full=is_full, v_proj=v_proj, seed=7, kv_ring_mask=ring)
+    rig = QR.RopeRig(f)
+    q0, k0 = rig.buf_q.clone(), rig.buf_k.clone()
+    # correctness first, against the oracle with the reference's storage rounding
+    rig.run_dispatch()
+    tr = lambda x: R.bf16_bits_to_f32(R.f32_to_bf16_bits_trunc(x))
+    od = po.make_rope_desc(canvas, nq, nkv, hd, kv_len, is_full=is_full, v_from_k=(v_proj == 0), kv_ring_mask=ring)
+    t_cpu = time.perf_counter()
+    rq, rk, rkv = po.qk_rope_kv_f32(od, tr(f.q), tr(f.k), tr(f.v), f.kvcache, tr(f.q_norm_w), tr(f.k_norm_w))
+    t_cpu = time.perf_counter() - t_cpu
+    gq, gk, gkv = rig.read()
+    err_q = float(np.max(np.abs(gq - tr(rq)) - np.abs(rq) * 2.0 ** -7))
+    err_kv = float(np.max(np.abs(gkv - R.f16_bits_to_f32(R.f32_to_f16_bits_trunc(rkv))) - np.abs(rkv) * 2.0 ** -10))
+    check = {"max_abs_beyond_one_storage_step": {"q": err_q, "kvcache": err_kv}, "tol": 1e-2,
+             "passed": bool(err_q <= 1e-2 and err_kv <= 1e-2 and np.isfinite(gq).all() and np.isfinite(gkv).all())}
+    # bytes every launch has to move: q read + written, k and v read (k twice when V aliases it: once per
+    # head that reads it), k written back unless aliased, the canvas rows of the cache written
+    eb = 2
+    nbytes = 2 * canvas * nq * hd * eb + canvas * nkv * hd * eb * (2 if v_proj == 0 else 3) + 2 * canvas * nkv * hd * eb
+    L, P, dims = QR.layer_offsets(f), A.step_params(kv_len), capi.AttnDims(canvas, nq, 0, 0)
+    lib = capi.load()
+
+    def step():
+        capi.check(lib.dg_qk_rope_kv_dispatch(rig.buf_q.data_ptr(), rig.buf_k.data_ptr(), rig.buf_v.data_ptr(),
+                                              rig.buf_kv.data_ptr(), rig.buf_blob.data_ptr(), C.byref(L), C.byref(P),
+                                              C.byref(dims), None, A.stream_handle()))
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms = (t1 - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps       # back-to-back launches of this one kernel on the stream
+    res = {"metric": "qk_rope_kv (RMSNorm + RoPE + KV write) GB/s, one layer, 256-row canvas @ 32k prefix, 1 GPU",
+           "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+           "data": "synthetic",
+           "config": {"workload": args.workload, "canvas": canvas, "n_q_heads": nq, "n_kv_heads": nkv, "head_dim": hd,
+                      "kv_prefix": kv_len, "is_full": is_full, "v_from_k": v_proj == 0, "kv_ring_mask": ring,
+                      "cache": "f16, reference slot-major layout"},
+           "bytes_per_step": nbytes,
+           "roofline": {"bound": "hbm", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": nbytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "kernel": "qk_rope_kv_kernel", "kernel_ms": kern_ms},
+           "cpu_baseline": {"value": nbytes / t_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                            "sample": f"the whole launch once, {t_cpu:.3f} s, scalar restatement of the reference CPU twin"},
+           "check": check}
+    print(json.dumps(res), flush=True)
+    if not check["passed"]:
+        sys.exit(1)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -92,6 +162,10 @@ def main():
         torch.cuda.synchronize()
         assert torch.equal(src, dst)
         print(json.dumps({"calib_copy_bytes": nbytes, "launches": args.steps, "kernel": "calib_copy_kernel"}))
+        return
+
+    if args.workload in PRODUCER_SHAPES:
+        bench_producer(args)
         return
 
     w = W.config(args.workload)

@@ -4,8 +4,8 @@
 //
 // One wave per (canvas row, head), heads = Hq query heads, then Hkv key heads, then Hkv value
 // heads, exactly the reference's grid (enc.rs:1794-1804).  The row (at most 1 KiB) is read once
-// with 16-byte loads, normalised in registers, staged in LDS so the rotation can pair element d
-// with its partner, and written once: Q (and K, unless V aliases it) back in place as bf16, K
+// with up to 16-byte loads, normalised in registers, staged in LDS where each lane rotates one
+// pair (d, hd/2 + d) per pass (one sincos per pair), and written once: Q (and K, unless V aliases it) back in place as bf16, K
 // and V into the cache at slot(pos) in the cache's element type.  HBM-bound by construction:
 // every byte moves once; at 256 canvas rows the launch is a few megabytes, i.e. latency-bound.
 #include "attn_params.h"
@@ -44,19 +44,62 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-__device__ __forceinline__ void store_cache(void* base, uint32_t dt, int64_t idx, float v) {
-  if (dt == DT_F16) ((_Float16*)base)[idx] = (_Float16)v;           // kv_store: half(v), round to nearest
-  else ((uint16_t*)base)[idx] = f32_to_bf16_bits(v, false);
-}
-
 constexpr float kRmsEps = 1e-6f;   // cpu.rs:3, attention_device.metal:10
 
+// One row of `hd` bf16 elements, `per` = hd/64 consecutive ones per lane, moved with the widest
+// access the count allows (16 bytes at hd 512).
+template <int PER>
+__device__ __forceinline__ void load_row(const uint16_t* src, float (&x)[8]) {
+  if constexpr (PER == 8) {
+    const uint4 r = *(const uint4*)src;
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __uint_as_float(w[i] << 16);
+      x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  } else if constexpr (PER == 4) {
+    const uint2 r = *(const uint2*)src;
+    x[0] = __uint_as_float(r.x << 16);
+    x[1] = __uint_as_float(r.x & 0xffff0000u);
+    x[2] = __uint_as_float(r.y << 16);
+    x[3] = __uint_as_float(r.y & 0xffff0000u);
+  } else if constexpr (PER == 2) {
+    const uint32_t r = *(const uint32_t*)src;
+    x[0] = __uint_as_float(r << 16);
+    x[1] = __uint_as_float(r & 0xffff0000u);
+  } else {
+    x[0] = bf16_bits_to_f32(src[0]);
+  }
+}
+
+// `per` consecutive elements as 16-bit storage values, packed and written with one store
+template <int PER>
+__device__ __forceinline__ void store_row16(uint16_t* dst, const uint16_t (&h)[8]) {
+  if constexpr (PER == 8) {
+    *(uint4*)dst = make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16,
+                              h[6] | (uint32_t)h[7] << 16);
+  } else if constexpr (PER == 4) {
+    *(uint2*)dst = make_uint2(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16);
+  } else if constexpr (PER == 2) {
+    *(uint32_t*)dst = h[0] | (uint32_t)h[1] << 16;
+  } else {
+    dst[0] = h[0];
+  }
+}
+
+__device__ __forceinline__ uint16_t cache_bits(uint32_t dt, float v) {
+  if (dt == DT_F16) return __builtin_bit_cast(uint16_t, (_Float16)v);   // kv_store: half(v), round to nearest
+  return f32_to_bf16_bits(v, false);
+}
+
+template <int PER>
 __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   __shared__ float stage[4][512];
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t tok = blockIdx.x, h = blockIdx.y * 4 + wave;
   const uint32_t n_heads = p.hq + 2 * p.hkv;
-  if (h >= n_heads) return;   // whole wave leaves; no barrier below involves it
+  if (h >= n_heads) return;   // the whole wave leaves; nothing below synchronises across waves
   const uint32_t hd = p.hd;
   const bool is_q = h < p.hq, is_k = !is_q && h < p.hq + p.hkv;
   const uint32_t hh = is_q ? h : (h - p.hq) % p.hkv;
@@ -68,76 +111,64 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   const uint16_t* src = (is_q || is_k) ? row_inplace
                                        : (p.v_from_k ? p.k : p.v) + ((size_t)tok * p.hkv + hh) * hd;
 
-  // lane owns elements [per*lane, per*lane + per), per = hd/64 (1 element for the first hd lanes if hd < 64)
-  const uint32_t per = hd >= 64 ? hd / 64 : 1;
-  const uint32_t d0 = lane * per;
+  // lane owns elements [PER*lane, PER*lane + PER); at hd < 64 only the first hd lanes own one
+  const uint32_t d0 = lane * PER;
   const bool active = d0 < hd;
-  float x[8];
+  float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (active) load_row<PER>(src + d0, x);
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    x[i] = 0.f;
-    if (active && (uint32_t)i < per) {
-      x[i] = bf16_bits_to_f32(src[d0 + i]);
-      ss += x[i] * x[i];
-    }
-  }
+  for (int i = 0; i < PER; ++i) ss += x[i] * x[i];
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)hd + kRmsEps);
-  if (lane == 0 && !(inv == inv && fabsf(inv) != INFINITY)) dbg_report(p.dbg, DG_DBG_ROPE_NONFINITE, (tok << 16) | h, __float_as_uint(inv));
+  if (lane == 0 && !(inv == inv && fabsf(inv) != INFINITY))
+    dbg_report(p.dbg, DG_DBG_ROPE_NONFINITE, (tok << 16) | h, __float_as_uint(inv));
 
+  uint16_t bits[8];
   if (!is_q && !is_k) {   // V: normalise without weight, write to the cache (cpu.rs:110-122)
     if (kv_write && active) {
-      const int64_t base = slot * p.v_tok_stride + (int64_t)hh * p.v_head_stride;
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if ((uint32_t)i < per) store_cache(p.vc, p.kv_dtype, base + d0 + i, x[i] * inv);
+      for (int i = 0; i < PER; ++i) bits[i] = cache_bits(p.kv_dtype, x[i] * inv);
+      store_row16<PER>((uint16_t*)p.vc + slot * p.v_tok_stride + (int64_t)hh * p.v_head_stride + d0, bits);
     }
     return;
   }
 
-  const uint16_t* w = is_q ? p.qw : p.kw;
   float* st = stage[wave];
+  if (active) {
+    float w[8];
+    load_row<PER>((is_q ? p.qw : p.kw) + d0, w);
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
-    if (active && (uint32_t)i < per) {
-      x[i] *= inv * bf16_bits_to_f32(w[d0 + i]);   // x * (inv * w), the CPU twin's order (cpu.rs:71-74)
-      st[d0 + i] = x[i];
-    }
+    for (int i = 0; i < PER; ++i) st[d0 + i] = x[i] * (inv * w[i]);   // x * (inv * w), the CPU twin's order (cpu.rs:71-74)
+  }
   __builtin_amdgcn_wave_barrier();   // the stage is private to the wave, whose LDS operations execute in order
 
-  // rotation (cpu.rs:31-65): split-half pairs (d, d + rot/2) over the whole head with theta 1e4;
-  // proportional pairs (d, hd/2 + d) for d < rot/2 = hd/8 with theta 1e6, the rest is left alone
-  const uint32_t half_rot = p.is_full ? hd / 8 : hd / 2;
-  const uint32_t partner_off = hd / 2;     // both schemes pair d with d + hd/2 (split-half: rot/2 = hd/2)
+  // rotation (cpu.rs:31-65): pairs (d, hd/2 + d) for d < rot/2; split-half: rot = hd, theta 1e4;
+  // proportional: rot = hd/4, theta 1e6, everything else is left alone.  One pair per lane and pass.
+  const uint32_t half_rot = p.is_full ? hd / 8 : hd / 2, off = hd / 2;
+  for (uint32_t dd = lane; dd < half_rot; dd += 64) {
+    const float a = (float)pos * p.inv_freq[dd];
+    float s, c;
+    sincosf(a, &s, &c);
+    const float x0 = st[dd], x1 = st[dd + off];
+    st[dd] = x0 * c - x1 * s;
+    st[dd + off] = x0 * s + x1 * c;
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (!active) return;
   float y[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    y[i] = x[i];
-    if (active && (uint32_t)i < per) {
-      const uint32_t d = d0 + i;
-      const bool first = d < half_rot, second = d >= partner_off && d < partner_off + half_rot;
-      if (first || second) {
-        const uint32_t dd = first ? d : d - partner_off;
-        const float a = (float)pos * p.inv_freq[dd];
-        const float c = cosf(a), s = sinf(a);
-        const float x0 = st[dd], x1 = st[dd + partner_off];
-        y[i] = first ? x0 * c - x1 * s : x0 * s + x1 * c;
-      }
-    }
-  }
-  if (!active) return;
+  for (int i = 0; i < PER; ++i) y[i] = st[d0 + i];
   if (is_k && kv_write) {
-    const int64_t base = slot * p.k_tok_stride + (int64_t)hh * p.k_head_stride;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      if ((uint32_t)i < per) store_cache(p.kc, p.kv_dtype, base + d0 + i, y[i]);
+    for (int i = 0; i < PER; ++i) bits[i] = cache_bits(p.kv_dtype, y[i]);
+    store_row16<PER>((uint16_t*)p.kc + slot * p.k_tok_stride + (int64_t)hh * p.k_head_stride + d0, bits);
   }
   // Q always goes back in place; K only when V does not alias the raw k projection (cpu.rs:137-143)
   if (is_q || !p.v_from_k) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      if ((uint32_t)i < per) row_inplace[d0 + i] = f32_to_bf16_bits(y[i], p.qk_trunc != 0);
+    for (int i = 0; i < PER; ++i) bits[i] = f32_to_bf16_bits(y[i], p.qk_trunc != 0);
+    store_row16<PER>(row_inplace + d0, bits);
   }
 }
 
@@ -189,7 +220,21 @@ int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* 
   const uint32_t half_rot = d->is_full ? hd / 8 : hd / 2;  // rot = hd/4 or hd (cpu.rs:17-23)
   for (uint32_t dd = 0; dd < half_rot; ++dd) p.inv_freq[dd] = std::pow(theta, -2.0f * (float)dd / (float)hd);
   const uint32_t n_heads = d->n_q_heads + 2 * d->n_kv_heads;
-  hipLaunchKernelGGL(dg::qk_rope_kv_kernel, dim3(d->canvas, (n_heads + 3) / 4), dim3(256), 0, (hipStream_t)stream, p);
+  // vector accesses of `per` elements: rows and the cache region must be aligned to them
+  const uint32_t per = hd >= 64 ? hd / 64 : 1;
+  const uintptr_t align = 2 * per;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)p.kc | (uintptr_t)p.vc | (uintptr_t)q_norm_w | (uintptr_t)k_norm_w |
+       (d->v_from_k ? 0 : (uintptr_t)v)) % align != 0)
+    return DG_ERR_LAYOUT;
+  if ((d->k_tok_stride | d->k_head_stride | d->v_tok_stride | d->v_head_stride) % per != 0) return DG_ERR_LAYOUT;
+  const dim3 grid(d->canvas, (n_heads + 3) / 4), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  switch (per) {
+    case 8: hipLaunchKernelGGL(dg::qk_rope_kv_kernel<8>, grid, block, 0, s, p); break;
+    case 4: hipLaunchKernelGGL(dg::qk_rope_kv_kernel<4>, grid, block, 0, s, p); break;
+    case 2: hipLaunchKernelGGL(dg::qk_rope_kv_kernel<2>, grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL(dg::qk_rope_kv_kernel<1>, grid, block, 0, s, p); break;
+  }
   return hipGetLastError() == hipSuccess ? DG_OK : DG_ERR_LAUNCH;
 }
 
