@@ -139,6 +139,129 @@ def bench_producer(args):
         sys.exit(1)
 
 
+def bench_schedule(args):
+    """One step = one denoise iteration of the 30-layer stack at prefix 32768: per layer the producer
+    (RMSNorm + RoPE + KV write of the 256 canvas rows) and the attention call, captured once in a HIP
+    graph and replayed.  25 sliding layers (Hkv 8, hd 256, window 1024 on a 2048-slot ring) and 5 global
+    layers (Hkv 2, hd 512) at indices 5, 11, 17, 23, 29; the canvas projections are regenerated on the
+    device before every iteration, the prefix rows stay."""
+    import torch
+    from diffgemma_amd import attention as A, capi, qk_rope_kv as QR, rounding as R, step_kv
+    from oracle import pyoracle as po
+    canvas, nq, kv_len, ring = 256, 16, 32768, 2048
+    lib = capi.load()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1234)
+
+    def unit_rows(n, hd):      # rows with unit RMS, bf16 bits: what a cache holds after the producer
+        x = torch.randn(n, hd, device="cuda", generator=gen)
+        x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+        return x.to(torch.bfloat16).view(torch.int16).reshape(-1)
+
+    layers, flops_iter = [], 0.0
+    for i in range(step_kv.N_LAYERS):
+        full = i in step_kv.FULL_LAYERS
+        hd, nkv = (512, 2) if full else (256, 8)
+        slots = kv_len + canvas if full else ring
+        mask = 0 if full else ring - 1
+        f = QR.random_fixture(1, nq, nkv, hd, kv_len, is_full=full, v_proj=0 if full else 1, seed=100 + i,
+                              kv_ring_mask=mask)      # norm weights and flags only; the buffers are made below
+        f.canvas = canvas
+        rd = QR.rope_desc(f, kv_dtype=capi.DG_BF16, truncate=False, layout="head_major", t_cap=slots)
+        ad = A.make_desc(canvas, nq, nkv, hd, kv_len, window=0 if full else 1024, kv_ring_mask=mask,
+                         q_dtype=capi.DG_BF16, kv_dtype=capi.DG_BF16, out_dtype=capi.DG_BF16, layout="head_major",
+                         t_cap=slots)
+        lay = {"full": full, "hd": hd, "nkv": nkv, "rd": rd, "ad": ad,
+               "cache": unit_rows(2 * nkv * slots, hd),         # every slot live: prefix rows (ring: its window)
+               "q": torch.empty(canvas * nq * hd, dtype=torch.int16, device="cuda"),
+               "k": torch.empty(canvas * nkv * hd, dtype=torch.int16, device="cuda"),
+               "v": torch.empty(canvas * nkv * hd, dtype=torch.int16, device="cuda"),
+               "qw": A.to_device_bits(R.f32_to_bf16_bits_rne(f.q_norm_w)),
+               "kw": A.to_device_bits(R.f32_to_bf16_bits_rne(f.k_norm_w)),
+               "out": torch.zeros(canvas * nq * hd, dtype=torch.int16, device="cuda"),
+               "ws": A.alloc_workspace(ad)}
+        layers.append(lay)
+        flops_iter += capi.visible_pairs(ad)[1]
+
+    def regenerate(it):        # canvas projections of iteration `it`: N(0, 1), device RNG keyed by seed + iteration
+        gen.manual_seed(5678 + it)
+        for lay in layers:
+            for name in ("q", "k", "v"):
+                t = lay[name]
+                t.copy_(torch.randn(t.numel(), device="cuda", generator=gen).to(torch.bfloat16).view(torch.int16))
+
+    def encode():              # what one denoise iteration enqueues for attention, layer by layer
+        st = A.stream_handle()
+        for lay in layers:
+            capi.check(lib.dg_qk_rope_kv(C.byref(lay["rd"]), lay["q"].data_ptr(), lay["k"].data_ptr(),
+                                         lay["v"].data_ptr(), lay["cache"].data_ptr(), lay["qw"].data_ptr(),
+                                         lay["kw"].data_ptr(), None, st))
+            A.forward(lay["ad"], lay["q"], lay["cache"], lay["out"], None, lay["ws"])
+
+    regenerate(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        encode()               # eager pass on the capture stream first
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager_out = [lay["out"].clone() for lay in layers]
+    graph = torch.cuda.CUDAGraph()
+    regenerate(0)              # the producer rotated q in place: same inputs again for the captured pass
+    with torch.cuda.graph(graph):
+        encode()
+    graph.replay()
+    torch.cuda.synchronize()
+    replay_equals_eager = all(torch.equal(a, lay["out"]) for a, lay in zip(eager_out, layers))
+
+    # parity of one layer of each kind against the oracle, on the inputs the device holds after the producer
+    check = {"replay_equals_eager": bool(replay_equals_eager), "layers": {}}
+    ok = replay_equals_eager
+    for idx in (0, 5):
+        lay = layers[idx]
+        hd, nkv, slots = lay["hd"], lay["nkv"], (kv_len + canvas if lay["full"] else ring)
+        qh = R.bf16_bits_to_f32(lay["q"].cpu().numpy().view(np.uint16))
+        kvh = R.bf16_bits_to_f32(lay["cache"].cpu().numpy().view(np.uint16))
+        od = po.make_desc(canvas, nq, nkv, hd, kv_len, window=0 if lay["full"] else 1024,
+                          kv_ring_mask=0 if lay["full"] else ring - 1, layout="head_major", t_cap=slots)
+        toks = np.array([0, 100, 255], dtype=np.uint32)
+        ref, _ = po.attention_f32(od, qh, kvh, tok_list=toks)
+        got = R.bf16_bits_to_f32(lay["out"].cpu().numpy().view(np.uint16)).reshape(canvas, nq, hd)
+        d = np.abs(got[toks] - ref[toks])
+        check["layers"][str(idx)] = {"max_abs": float(d.max()), "mean_abs": float(d.mean())}
+        ok = ok and d.max() <= 2e-2 and d.mean() <= 2e-3 and np.isfinite(got).all()
+    check["tol"] = {"max_abs": 2e-2, "mean_abs": 2e-3}
+    check["passed"] = bool(ok)
+
+    for it in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(2 * args.steps)]
+    t_total = 0.0
+    for it in range(args.steps):
+        regenerate(it)         # outside the timed part: it stands in for the projections that precede attention
+        marks[2 * it].record()
+        graph.replay()
+        marks[2 * it + 1].record()
+    torch.cuda.synchronize()
+    per_iter = sorted(marks[2 * i].elapsed_time(marks[2 * i + 1]) for i in range(args.steps))
+    ms = sum(per_iter) / len(per_iter)
+    res = {"metric": "denoise attention, 30-layer stack (25 sliding + 5 global) @ 32k prefix: TFLOP/s of producer + "
+                     "attention per denoise iteration, HIP graph replay, 1 GPU",
+           "value": flops_iter / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "cfg5_schedule", "layers": step_kv.N_LAYERS, "global_layers": list(step_kv.FULL_LAYERS),
+                      "canvas": canvas, "kv_prefix": kv_len, "sliding": "Hq16/Hkv8 hd256 window 1024 ring 2048",
+                      "global": "Hq16/Hkv2 hd512", "kv_layout": "bf16 head-major planes", "launch": "HIP graph, 120 kernels"},
+           "flops_per_step": flops_iter, "canvas_tokens_per_s": canvas / (ms * 1e-3),
+           "iteration_ms": {"min": per_iter[0], "median": per_iter[len(per_iter) // 2], "max": per_iter[-1]},
+           "roofline": None, "cpu_baseline": None, "check": check}
+    print(json.dumps(res), flush=True)
+    if not check["passed"]:
+        sys.exit(1)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -166,6 +289,9 @@ def main():
 
     if args.workload in PRODUCER_SHAPES:
         bench_producer(args)
+        return
+    if args.workload == "cfg5_schedule":
+        bench_schedule(args)
         return
 
     w = W.config(args.workload)

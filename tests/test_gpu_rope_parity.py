@@ -161,3 +161,70 @@ def test_rejects_bad_arguments(gpu_ready):
     d = QR.rope_desc(f)
     d.kv_ring_mask = 5
     assert lib.dg_qk_rope_kv(C.byref(d), *args) == capi.DG_ERR_LAYOUT
+
+
+def test_two_layer_step_in_a_hip_graph(gpu_ready, po):
+    """Producer + attention of a sliding (ring) and a global layer captured once and replayed with
+    regenerated canvas projections: every replay equals the eager result for the same inputs."""
+    import torch
+    canvas, nq, kv_len, ring = 64, 16, 3000, 2048
+    lib = capi.load()
+    gen = torch.Generator(device="cuda")
+    layers = []
+    for full in (False, True):
+        hd, nkv = (512, 2) if full else (256, 8)
+        slots = kv_len + canvas if full else ring
+        mask = 0 if full else ring - 1
+        f = QR.random_fixture(1, nq, nkv, hd, kv_len, is_full=full, v_proj=0 if full else 1, seed=3, kv_ring_mask=mask)
+        f.canvas = canvas
+        rd = QR.rope_desc(f, kv_dtype=capi.DG_BF16, truncate=False, layout="head_major", t_cap=slots)
+        ad = A.make_desc(canvas, nq, nkv, hd, kv_len, window=0 if full else 1024, kv_ring_mask=mask,
+                         q_dtype=capi.DG_BF16, kv_dtype=capi.DG_BF16, out_dtype=capi.DG_BF16, layout="head_major",
+                         t_cap=slots)
+        gen.manual_seed(11)
+        cache = torch.randn(2 * nkv * slots * hd, device="cuda", generator=gen).to(torch.bfloat16).view(torch.int16)
+        layers.append(dict(rd=rd, ad=ad, cache=cache, ws=A.alloc_workspace(ad),
+                           q=torch.empty(canvas * nq * hd, dtype=torch.int16, device="cuda"),
+                           k=torch.empty(canvas * nkv * hd, dtype=torch.int16, device="cuda"),
+                           v=torch.empty(canvas * nkv * hd, dtype=torch.int16, device="cuda"),
+                           qw=A.to_device_bits(R.f32_to_bf16_bits_rne(f.q_norm_w)),
+                           kw=A.to_device_bits(R.f32_to_bf16_bits_rne(f.k_norm_w)),
+                           out=torch.zeros(canvas * nq * hd, dtype=torch.int16, device="cuda")))
+
+    def regenerate(it):
+        gen.manual_seed(100 + it)
+        for lay in layers:
+            for n in ("q", "k", "v"):
+                lay[n].copy_(torch.randn(lay[n].numel(), device="cuda", generator=gen).to(torch.bfloat16).view(torch.int16))
+
+    def encode():
+        for lay in layers:
+            capi.check(lib.dg_qk_rope_kv(C.byref(lay["rd"]), lay["q"].data_ptr(), lay["k"].data_ptr(), lay["v"].data_ptr(),
+                                         lay["cache"].data_ptr(), lay["qw"].data_ptr(), lay["kw"].data_ptr(), None,
+                                         A.stream_handle()))
+            A.forward(lay["ad"], lay["q"], lay["cache"], lay["out"], None, lay["ws"])
+
+    regenerate(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        encode()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    regenerate(0)
+    with torch.cuda.graph(g):
+        encode()
+    for it in range(1, 4):
+        regenerate(it)
+        encode()                                   # eager, on the same inputs
+        torch.cuda.synchronize()
+        want = [lay["out"].clone() for lay in layers]
+        regenerate(it)                             # the producer rotated q in place: restore the inputs
+        for lay in layers:
+            lay["out"].zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        for w, lay in zip(want, layers):
+            assert torch.equal(w, lay["out"]), it
+            assert np.isfinite(R.bf16_bits_to_f32(lay["out"].cpu().numpy().view(np.uint16))).all()
