@@ -372,15 +372,18 @@ def main():
     traffic = MEASURED_HBM_BYTES_PER_LAUNCH.get(args.workload)
 
     res = {
-        "metric": "denoise attention TFLOP/s + % bf16 MFMA peak, 256-canvas @ 32k prefix, 1 GPU",
+        "metric": ("denoise attention TFLOP/s + % bf16 MFMA peak, 256-canvas @ 32k prefix, 1 GPU"
+                   if not w.name.startswith("prefill_") else
+                   f"causal prefill attention TFLOP/s, {w.canvas}-row super-chunk @ {w.kv_len} prefix, 1 GPU"),
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if w.dtype == "bf16" else "f16", "data": "synthetic",
         "config": {"workload": w.name, "canvas": w.canvas, "kv_prefix": w.kv_len, "n_q_heads": w.n_q_heads,
                    "n_kv_heads": w.n_kv_heads, "head_dim": w.head_dim, "causal_rows": w.causal_rows,
                    "window": w.window, "kv_layout": w.layout, "n_splits": n_splits,
-                   "mask": "rows<causal_rows causal in canvas, rest bidirectional; prefix all-visible"
-                           if not w.window else "sliding window, reference rule t_lo=kv_len-(window-1)"},
+                   "mask": ("every row causal (prefill): keys [max(0, pos-(window-1)), pos]" if w.causal_rows == w.canvas
+                            else "rows<causal_rows causal in canvas, rest bidirectional; prefix all-visible"
+                            if not w.window else "sliding window, reference rule t_lo=kv_len-(window-1)")},
         "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "canvas_tokens_per_s": w.canvas / (ms_per_step * 1e-3),
         "flops_per_step": flops, "visible_pairs_per_head": pairs,

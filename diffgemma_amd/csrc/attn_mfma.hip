@@ -395,17 +395,20 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   float* const sml = (float*)(smem + OFF_ML);
 
   // ---- which (KV head, split, row tile) this workgroup owns ----
-  // Workgroup ids go round-robin over the 8 XCDs.  All row tiles of one (KV head, split)
-  // stream the same keys, so they are given ids with the same id%8 and share one L2.
-  const uint32_t nstream = p.hkv * p.n_splits;
+  // Workgroup ids go round-robin over the 8 XCDs, each with its own L2.  The units, ordered
+  // (KV head, split) first and row tile second, are cut into 8 equal runs, one per XCD, so the
+  // row tiles that stream the same keys sit behind one L2 and every XCD has work whatever
+  // the number of (KV head, split) pairs.
+  const uint32_t n_units = p.hkv * p.n_splits * p.n_mtiles;
+  const uint32_t per_xcd = (n_units + 7u) >> 3;
   const uint32_t wg = blockIdx.x;
-  const uint32_t slot_in_xcd = wg >> 3;
+  const uint32_t unit = (wg & 7u) * per_xcd + (wg >> 3);
+  if (unit >= n_units) return;
   // (the divisions by run-time values are done by the vector unit; readfirstlane tells the
   // compiler the results are the same in every lane, so everything derived from them stays in
   // scalar registers)
-  const uint32_t stream = __builtin_amdgcn_readfirstlane((slot_in_xcd / p.n_mtiles) * 8u + (wg & 7u));
-  const uint32_t mt = __builtin_amdgcn_readfirstlane(slot_in_xcd % p.n_mtiles);
-  if (stream >= nstream) return;
+  const uint32_t stream = __builtin_amdgcn_readfirstlane(unit / p.n_mtiles);
+  const uint32_t mt = __builtin_amdgcn_readfirstlane(unit % p.n_mtiles);
   const uint32_t kvh = __builtin_amdgcn_readfirstlane(stream / p.n_splits);
   const uint32_t split = __builtin_amdgcn_readfirstlane(stream % p.n_splits);
 
@@ -452,10 +455,13 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     hi_min = __builtin_amdgcn_readfirstlane(hi_min);
     hi_max = __builtin_amdgcn_readfirstlane(hi_max);
   }
-  const uint32_t split_begin = p.tile_first + split * p.tiles_per_split;
-  const uint32_t split_end = min(split_begin + p.tiles_per_split, p.tile_end);
-  const uint32_t tb = __builtin_amdgcn_readfirstlane(max(lo_min / kBlockN, split_begin));
-  const uint32_t te = __builtin_amdgcn_readfirstlane(min((hi_max + kBlockN - 1) / kBlockN, split_end));
+  // the key tiles this row tile can see, cut into n_splits equal runs (a causal or windowed row
+  // tile sees only part of the launch's key range: cutting its own range keeps the splits even)
+  const uint32_t mt_begin = max(lo_min / kBlockN, p.tile_first);
+  const uint32_t mt_end = max(min((hi_max + kBlockN - 1) / kBlockN, p.tile_end), mt_begin);
+  const uint32_t per_split = (mt_end - mt_begin + p.n_splits - 1u) / p.n_splits;
+  const uint32_t tb = __builtin_amdgcn_readfirstlane(min(mt_begin + split * per_split, mt_end));
+  const uint32_t te = __builtin_amdgcn_readfirstlane(min(tb + per_split, mt_end));
   const uint32_t ntile = te > tb ? te - tb : 0u;
 
   // ---- Q fragments: B operand of S^T = K.Q^T, lane = row, 8 consecutive d per step ----
@@ -878,7 +884,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 template <int D, bool F16>
 hipError_t launch_one(const AttnParams& p, hipStream_t s) {
   const uint32_t nstream = p.hkv * p.n_splits;
-  const uint32_t grid = ((nstream + 7u) / 8u) * p.n_mtiles * 8u;
+  const uint32_t grid = ((nstream * p.n_mtiles + 7u) / 8u) * 8u;
   hipLaunchKernelGGL((attn_mfma_kernel<D, F16>), dim3(grid), dim3(256), 0, s, p);
   return hipGetLastError();
 }

@@ -77,6 +77,14 @@ def config(name: str) -> Workload:
                         outlier_gain=8.0, seed=4)
     if name == "cfg5_sliding_32k":    # sliding layer of the 30-layer schedule at prefix 32768
         return Workload(name, 256, 16, 8, 256, 32768, window=1024, seed=5)
+    # causal extend of the committed prefix by 4 x 256 tokens in one call (the reference's batched
+    # prefill super-chunk, src/metal/step_kernel/runtime.rs:370-389, enc.rs:2576-2585)
+    if name == "prefill_global_super":
+        return Workload(name, 1024, 16, 2, 512, 32768, causal_rows=1024, seed=6)
+    if name == "prefill_sliding_super":
+        return Workload(name, 1024, 16, 8, 256, 32768, causal_rows=1024, window=1024, seed=7)
+    if name == "prefill_global_fresh":    # first super-chunk of a prompt: no prefix, triangular mask
+        return Workload(name, 1024, 16, 2, 512, 0, causal_rows=1024, seed=8)
     raise KeyError(name)
 
 

@@ -257,6 +257,29 @@ def test_causal_rows_equal_all_valid_on_prefix(po):
     assert max_abs_diff(wc[0], wa[0]) > 1e-4 and np.array_equal(wc[-1], wa[-1])
 
 
+@pytest.mark.parametrize("window", [0, 5, 11])
+def test_causal_super_chunk_is_its_sub_chunks(po, window):
+    """A causal call over n_subs * c rows at kv_len == the per-sub-chunk calls the reference encodes
+    (rows [s*c, (s+1)*c) at kv_len + s*c; src/metal/step_kernel/runtime.rs:370-389), and every row
+    with a window is the dense result over keys [pos-(window-1), pos]."""
+    rng = np.random.default_rng(5)
+    c, subs, hq, hkv, hd, kvl = 4, 3, 4, 2, 32, 9
+    canvas, t_all = c * subs, kvl + c * subs
+    q = rng.standard_normal((canvas, hq, hd)).astype(np.float32)
+    kv = rng.standard_normal((t_all, 2, hkv, hd)).astype(np.float32)
+    big, big_lse = po.attention_f32(po.make_desc(canvas, hq, hkv, hd, kvl, causal_rows=canvas, window=window), q, kv)
+    for s_ in range(subs):
+        d = po.make_desc(c, hq, hkv, hd, kvl + s_ * c, causal_rows=c, window=window)
+        out, lse = po.attention_f32(d, q[s_ * c:(s_ + 1) * c], kv[:kvl + (s_ + 1) * c])
+        assert np.array_equal(out, big[s_ * c:(s_ + 1) * c]) and np.array_equal(lse, big_lse[s_ * c:(s_ + 1) * c])
+    for r in range(canvas):
+        pos = kvl + r
+        lo = max(0, pos - (window - 1)) if window else 0
+        want, want_lse = dense_reference(q[r:r + 1], kv[lo:pos + 1, 0], kv[lo:pos + 1, 1], np.ones((1, pos + 1 - lo), bool))
+        assert max_abs_diff(big[r], want[0]) < 5e-6
+        assert np.max(np.abs(big_lse[r] - want_lse[0])) < 2e-5
+
+
 def test_mixed_mask_is_rowwise_composition(po):
     f = A.full_grp8_hd512_fixture()   # canvas 16
     cr = 6
