@@ -38,34 +38,10 @@
 // 2^tau * keys * |v|, far from 2^127 for tau = 80.  With f16 operands P itself has to stay
 // below 65504.
 #include "attn_params.h"
-
-#include <type_traits>
+#include "mfma_tile.h"
 
 namespace dg {
 namespace {
-
-// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N)
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
-}
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef short i16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-typedef __attribute__((address_space(3))) char lds_char;
-typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
-typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
-typedef __attribute__((address_space(1))) const void gbl_void;
-typedef __attribute__((address_space(3))) void lds_void;
 
 // log2 units by which a tile max may exceed the reference max before the reference is raised
 template <bool F16>
@@ -91,18 +67,6 @@ constexpr float kTau = F16 ? 12.0f : 80.0f;
 #define DG_PHASE_STORE
 #endif
 
-template <bool F16>
-__device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
-  if constexpr (F16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-  } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  }
-}
-
-// two floats -> packed pair of E (round to nearest even), low half = a
 // Score MFMAs, written as assembly so that their accumulator is an ordinary VGPR tuple.  O fills
 // all 256 accumulation registers at head_dim 512; the compiler gives every MFMA of such a
 // kernel an accumulation-register destination, which made it park one block of O in VGPRs
@@ -173,32 +137,6 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v) {
   return v;
 }
 
-template <bool F16>
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  if constexpr (F16) {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    h2 v = {(_Float16)a, (_Float16)b};
-    return __builtin_bit_cast(uint32_t, v);
-  } else {
-    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-    b2 v = {(__bf16)a, (__bf16)b};
-    return __builtin_bit_cast(uint32_t, v);
-  }
-}
-template <bool F16>
-__device__ __forceinline__ float unpack_lo(uint32_t u) {
-  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(u & 0xffffu));
-  else return __uint_as_float(u << 16);
-}
-template <bool F16>
-__device__ __forceinline__ float unpack_hi(uint32_t u) {
-  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(u >> 16));
-  else return __uint_as_float(u & 0xffff0000u);
-}
-
-// s_waitcnt vmcnt(0) as a builtin, so that the compiler's own wait-count bookkeeping sees it
-// (gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt = 6:4, lgkmcnt = 11:8; the other two
-// counters are left at their maxima).
 // acc + lo + hi of a packed pair, in one dot-product instruction
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
@@ -210,164 +148,6 @@ __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
   } else {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u),
                                            acc, false);
-  }
-}
-
-// wait until at most N of this wave's vector memory loads are outstanding (N <= 15)
-template <int N>
-__device__ __forceinline__ void wait_vmem_but() {
-  static_assert(N >= 0 && N <= 15, "vmcnt immediate");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
-}
-__device__ __forceinline__ void wait_vmem_all() {
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  asm volatile("" ::: "memory");
-}
-
-// value of lane l combined with lane l^32
-__device__ __forceinline__ float max_across_halves(float x) {
-  const uint32_t u = __float_as_uint(x);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float sum_across_halves(float x) {
-  const uint32_t u = __float_as_uint(x);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-// LDS layout of one 32-key tile of K or V (rows = keys, head_dim contiguous, 16-byte chunks).
-//
-// head_dim 512: a row is exactly the KiB one direct-to-LDS instruction writes, so rows can be
-// padded apart: K rows by 16 B (32 rows x one chunk per half-wave fall on distinct banks),
-// V rows by 64 B (the 8 rows x 4 chunks of a transposing read do).  Every fragment address is
-// then one per-lane base plus a compile-time offset, and the global side of a load is one
-// row: a scalar address plus lane*16.
-// smaller head_dim: several rows share an instruction's KiB, so rows stay dense and the 16-byte
-// chunks are XOR-swizzled instead (the swizzle is applied by choosing which global chunk each
-// lane fetches).
-template <int D>
-struct Lay {
-  static constexpr int CPR = D / 8;          // chunks per row
-  static constexpr int ROWB = 2 * D;         // bytes per row
-  static constexpr bool PAD = CPR == 64;
-  static constexpr int K_STRIDE = PAD ? ROWB + 16 : ROWB;
-  static constexpr int V_STRIDE = PAD ? ROWB + 64 : ROWB;
-  static constexpr int K_BYTES = 32 * K_STRIDE, V_BYTES = 32 * V_STRIDE;
-  static constexpr int NBLK = 32 * CPR / 64;   // KiB blocks (= load instructions) per tile
-  static constexpr int NLD = (NBLK + 3) / 4;   // load instructions per wave and tile
-  static __device__ __forceinline__ uint32_t swz_k(uint32_t row) {
-    if constexpr (PAD) return 0u;
-    else if constexpr (CPR >= 16) return row & 15u;
-    else return (row / (16 / CPR)) & (CPR - 1);
-  }
-  static __device__ __forceinline__ uint32_t swz_v(uint32_t row) {
-    if constexpr (PAD) return 0u;
-    else return ((row & 3u) << 2) & (CPR - 1);
-  }
-};
-
-// One tile's direct-to-LDS loads, described once per tile and issued one wave instruction at a
-// time so the issue slots can be spread between MFMAs.  Rows of the tile outside
-// [t_min, t_all) are replaced by the nearest row inside: those keys are masked for every query
-// row of the workgroup, but what their slots hold (dead ring slots, memory past the cache) may
-// not be finite, and 0 * NaN would poison P.V.
-struct TileLoad {
-  const char* base;   // head base + slot(t0) * row stride (wave-uniform)
-  uint32_t stride_b;  // bytes between key rows in global memory
-  uint32_t rmin;      // first row of the tile that may be read
-  uint32_t rmax;      // last row of the tile that may be read
-  uint32_t lds;       // LDS byte address of the destination buffer (padded layout: of this wave's first row)
-  // padded layout only, per lane: byte offsets from base of this lane's chunk in the first and
-  // the last row that may be read, and in the row of this wave's load 0
-  uint32_t lo_l, hi_l, raw0;
-};
-
-// FIRST: the tile may begin before t_min (only the first tile a workgroup visits can).
-template <int D, bool IS_V, bool FIRST>
-__device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_t tok_stride_b, uint32_t t0,
-                                                   uint32_t t_min, uint32_t t_all, uint32_t ring_mask, lds_char* buf,
-                                                   uint32_t wave, uint32_t lane) {
-  using L = Lay<D>;
-  TileLoad tl;
-  tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
-  tl.stride_b = (uint32_t)tok_stride_b;
-  tl.rmin = FIRST && t_min > t0 ? t_min - t0 : 0u;
-  tl.rmax = min(t_all - 1u - t0, (uint32_t)kBlockN - 1u);
-  tl.lds = (uint32_t)(size_t)buf;
-  if constexpr (L::PAD) {
-    tl.lds += wave * (IS_V ? L::V_STRIDE : L::K_STRIDE);
-    tl.lo_l = tl.rmin * tl.stride_b + lane * 16u;
-    tl.hi_l = tl.rmax * tl.stride_b + lane * 16u;
-    tl.raw0 = wave * tl.stride_b + lane * 16u;
-  }
-  return tl;
-}
-
-// The descriptor with every field computed at this point of the program (the compiler would
-// otherwise sink the arithmetic to the first use, which sits behind a branch where nothing
-// overlaps it).
-__device__ __forceinline__ TileLoad pinned(TileLoad tl) {
-  uint64_t b = (uint64_t)tl.base;
-  uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
-  uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
-  uint32_t lds = (uint32_t)__builtin_amdgcn_readfirstlane(tl.lds);
-  asm volatile("" : "+s"(lo), "+s"(hi), "+s"(lds), "+v"(tl.lo_l), "+v"(tl.hi_l), "+v"(tl.raw0));
-  tl.base = (const char*)(((uint64_t)hi << 32) | lo);
-  tl.lds = lds;
-  return tl;
-}
-
-// The loads are written as assembly on purpose: the compiler orders every LDS read after a
-// direct-to-LDS load it knows about with s_waitcnt vmcnt(0), which would expose the whole
-// fetch latency once per tile.  The kernel waits for these loads itself (wait_vmem_but).
-// All scalar operands are wave-uniform by construction; readfirstlane tells the compiler so
-// (it returns a signed int: without the casts the low half of the address would be
-// sign-extended over the high half).
-__device__ __forceinline__ uint64_t uniform_address(const char* base_uniform) {
-  const uint64_t b = (uint64_t)base_uniform;
-  return ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32) |
-         (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
-}
-// lane l: 16 bytes from base + voff -> LDS byte (lds_dst + LDS_IMM) + 16 * l
-template <int LDS_IMM>
-__device__ __forceinline__ void lds_dma_16(const char* base_uniform, uint32_t voff, uint32_t lds_dst_uniform) {
-  const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_dst_uniform);
-  const uint64_t base = uniform_address(base_uniform);
-  if constexpr (LDS_IMM == 0) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base)
-                 : "memory");
-  } else {
-    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff),
-                 "s"(base), "n"(LDS_IMM)
-                 : "memory", "scc");
-  }
-}
-
-template <int D, bool IS_V, int K>
-__device__ __forceinline__ void issue_tile_part(const TileLoad& tl, uint32_t wave, uint32_t lane) {
-  using L = Lay<D>;
-  if (L::NBLK < 4 && K * 4 + wave >= (uint32_t)L::NBLK) return;
-  if constexpr (L::PAD) {
-    // one instruction = one key row (row 4 K + wave): everything but the clamp of the row is
-    // either per tile or a compile-time constant
-    uint32_t voff;
-    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(voff) : "v"(tl.raw0 + (uint32_t)(4 * K) * tl.stride_b), "v"(tl.lo_l), "v"(tl.hi_l));
-    lds_dma_16<4 * K * (IS_V ? L::V_STRIDE : L::K_STRIDE)>(tl.base, voff, tl.lds);
-  } else {
-    const uint32_t blk = K * 4 + wave;
-    const uint32_t pch = blk * 64 + lane;
-    const uint32_t r = pch / L::CPR, pc = pch % L::CPR;
-    const uint32_t c = pc ^ (IS_V ? L::swz_v(r) : L::swz_k(r));
-    lds_dma_16<0>(tl.base, min(max(r, tl.rmin), tl.rmax) * tl.stride_b + c * 16u, tl.lds + blk * 1024u);
-  }
-}
-
-template <int D, bool IS_V, int K = 0>
-__device__ __forceinline__ void issue_tile(const TileLoad& tl, uint32_t wave, uint32_t lane) {
-  if constexpr (K < Lay<D>::NLD) {
-    issue_tile_part<D, IS_V, K>(tl, wave, lane);
-    issue_tile<D, IS_V, K + 1>(tl, wave, lane);
   }
 }
 

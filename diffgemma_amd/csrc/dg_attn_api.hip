@@ -136,6 +136,8 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
     lo_all = std::min(lo_all, (d->window && qpos0 > d->window - 1u) ? qpos0 - (d->window - 1u) : 0u);
   }
   lo_all = std::min(lo_all, pl->t_all);
+  // a ring must hold every visible position at once, or two of them share a slot
+  if (d->kv_ring_mask != 0 && pl->t_all - lo_all > d->kv_ring_mask + 1u) return DG_ERR_LAYOUT;
   pl->tile_first = lo_all / dg::kBlockN;
   pl->tile_end = (pl->t_all + dg::kBlockN - 1) / dg::kBlockN;
   const uint32_t ntiles = std::max(1u, pl->tile_end - pl->tile_first);

@@ -177,6 +177,74 @@ void dgo_attention_f32(const dgo_desc* dp, const float* q, const float* kv, floa
   }
 }
 
+// Top-k sparse attention: attention_topk/cpu.rs:41-120 (selection, tie-break, renormalised softmax,
+// summation in selection order) with the per-row k of attention_topk.metal:160-182.
+uint32_t dgo_topk_row_k(const uint32_t k_cfg[4], uint32_t n_valid, int causal_row) {
+  uint32_t k_req;
+  if (k_cfg[1] != 0u) {
+    const uint32_t gran = std::max(k_cfg[0], 1u);
+    const uint32_t t_equiv = causal_row ? ((n_valid + gran - 1u) / gran) * gran : n_valid;
+    k_req = std::min(std::max(t_equiv / k_cfg[1], k_cfg[2]), k_cfg[3]);
+  } else {
+    k_req = std::max(k_cfg[0], 1u);   // cpu.rs:59 (k.max(1))
+  }
+  return std::min(k_req, n_valid);
+}
+
+void dgo_attention_topk_f32(const dgo_desc* dp, const uint32_t k_cfg[4], const float* q, const float* kv, float* out,
+                            uint32_t* sel_idx, uint32_t sel_cap, uint32_t* sel_count, const uint32_t* tok_list,
+                            uint32_t n_tok, int n_threads) {
+  const dgo_desc d = *dp;
+  const uint32_t hd = d.head_dim, nq = d.n_q_heads, nkv = d.n_kv_heads;
+  const uint32_t group = nq / nkv;
+  const uint32_t t_all = d.kv_len + d.canvas;
+  const float scale = d.scale == 0.0f ? 1.0f : d.scale;
+  const uint32_t rows = tok_list ? n_tok : d.canvas;
+  const long units = (long)rows * nq;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads_or_all(n_threads))
+  for (long u = 0; u < units; ++u) {
+    const uint32_t tok = tok_list ? tok_list[u / nq] : (uint32_t)(u / nq);
+    const uint32_t qh = (uint32_t)(u % nq);
+    const uint32_t kvh = qh / group;
+    const RowRange r = row_range(d, tok);
+    const float* qv = q + ((size_t)tok * nq + qh) * hd;
+    float* o = out + ((size_t)tok * nq + qh) * hd;
+    // step 1: every valid score, a sequential fp32 dot product (cpu.rs:70-80)
+    std::vector<std::pair<float, uint32_t>> sc;
+    sc.reserve(t_all);
+    for (uint32_t t = 0; t < t_all; ++t) {
+      if (!vis(r, t, t_all)) continue;
+      const float* kk = kv + d.k_off + (int64_t)slot_of(d, t) * d.k_tok_stride + (int64_t)kvh * d.k_head_stride;
+      sc.emplace_back(dot_seq(qv, kk, hd) * scale, t);
+    }
+    const uint32_t n_valid = (uint32_t)sc.size();
+    const uint32_t kk_ = dgo_topk_row_k(k_cfg, n_valid, tok < d.causal_rows ? 1 : 0);
+    for (uint32_t i = 0; i < hd; ++i) o[i] = 0.0f;
+    if (sel_count) sel_count[(size_t)tok * nq + qh] = kk_;
+    if (kk_ == 0) continue;
+    // step 2: top-k by (score descending, index ascending) (cpu.rs:88-93)
+    std::partial_sort(sc.begin(), sc.begin() + kk_, sc.end(), [](const auto& a, const auto& b) {
+      return a.first > b.first || (a.first == b.first && a.second < b.second);
+    });
+    // step 3: softmax over the selected scores only (cpu.rs:95-104)
+    const float mmax = sc[0].first;
+    std::vector<float> probs(kk_);
+    float l = 0.0f;
+    for (uint32_t j = 0; j < kk_; ++j) {
+      probs[j] = std::exp(sc[j].first - mmax);
+      l += probs[j];
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    // step 4: weighted sum of the selected V rows, in selection order (cpu.rs:106-114)
+    for (uint32_t j = 0; j < kk_; ++j) {
+      const float pj = probs[j] * inv;
+      const float* vv = kv + d.v_off + (int64_t)slot_of(d, sc[j].second) * d.v_tok_stride + (int64_t)kvh * d.v_head_stride;
+      for (uint32_t i = 0; i < hd; ++i) o[i] += pj * vv[i];
+      if (sel_idx && j < sel_cap) sel_idx[((size_t)tok * nq + qh) * sel_cap + j] = sc[j].second;
+    }
+  }
+}
+
 void dgo_attention_f64(const dgo_desc* dp, const float* q, const float* kv, double* out, double* lse,
                        const uint32_t* tok_list, uint32_t n_tok, int n_threads) {
   const dgo_desc d = *dp;

@@ -14,6 +14,10 @@
  *   dgo_attention_bitmap_f32 src/model/attention.rs:354-394,861-934 + src/model/mask.rs:4-27
  *                            + src/shaders/cpu/mod.rs:175-190 (dense scores, MASK_NEG, softmax_rows)
  *   dgo_attention_f64        textbook two-pass softmax(QK^T)V in double (closed form, no reference twin)
+ *   dgo_attention_topk_f32   src/shaders/attn/attention_topk/cpu.rs:41-120 (exact top-k by f32 score, ties to the
+ *                            lower index, softmax over the kept keys, V summed in selection order);
+ *   dgo_topk_row_k           src/shaders/attn/attention_topk/attention_topk.metal:160-182 (fixed or
+ *                            context-adaptive k per row), src/flags/accessors.rs:210-221 (k_cfg)
  *   dgo_merge_partials_f32   closed form m=max m_i, l=sum l_i e^(m_i-m), O=sum O_i e^(m_i-m)/l; the
  *                            reference's state planes: attention_mma_full.metal:107-118,355-368
  *   rounding helpers         src/shaders/common/bf16.rs:9-41, src/shaders/common/f16.rs:3-60
@@ -39,6 +43,10 @@
  *     one-hot inputs show which elements are paired (split-half vs proportional) and which are
  *     left alone (proportional: only hd/4 of the head rotates); cache rows land at the slot the
  *     attention oracle reads; V = rms_norm_no_scale(raw k) when V aliases k
+ *   - top-k: k >= visible keys == the dense oracle; k = 1 == the V row of the arg-max key; numpy
+ *     brute force (lexsort by (-score, index), float64 softmax over the kept set) on random small
+ *     cases incl. duplicated keys (tie-break) and ragged causal rows (k > visible keys); the
+ *     per-row k rule against hand-computed values
  * LSE is not emitted anywhere in the reference; it is the closed form m + ln(l) of the
  * recurrence's own (m, l), cross-checked against a float64 logsumexp of the score row.
  */
@@ -83,6 +91,16 @@ uint64_t dgo_visible_pairs(const dgo_desc* d);
  * (may be NULL).  Only rows tok_list[0..n_tok) are computed when tok_list != NULL.  n_threads<=0: all. */
 void dgo_attention_f32(const dgo_desc* d, const float* q, const float* kv, float* out, float* lse,
                        const uint32_t* tok_list, uint32_t n_tok, int n_threads);
+/* Top-k sparse attention (attention_topk/cpu.rs:41-120): per (row, head) only the k highest scores among the
+ * visible keys are kept (ties: lower index first), softmax is renormalised over them and the V rows are summed
+ * in that order.  k_cfg = (fixed_k | chunk grid, dyn_divisor, k_min, k_max) as in attention_topk.metal:160-182:
+ * divisor 0 -> k = k_cfg[0]; else k = clamp(t_equiv / divisor, k_min, k_max) with t_equiv the row's visible-key
+ * count, rounded up to the grid for causal rows.  sel_idx [canvas][Hq][sel_cap] / sel_count [canvas][Hq] (may
+ * be NULL) receive the selected key positions in selection order. */
+uint32_t dgo_topk_row_k(const uint32_t k_cfg[4], uint32_t n_valid, int causal_row);
+void dgo_attention_topk_f32(const dgo_desc* d, const uint32_t k_cfg[4], const float* q, const float* kv, float* out,
+                            uint32_t* sel_idx, uint32_t sel_cap, uint32_t* sel_count, const uint32_t* tok_list,
+                            uint32_t n_tok, int n_threads);
 /* Same mask semantics, two-pass softmax in double. */
 void dgo_attention_f64(const dgo_desc* d, const float* q, const float* kv, double* out, double* lse,
                        const uint32_t* tok_list, uint32_t n_tok, int n_threads);

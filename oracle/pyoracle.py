@@ -60,6 +60,9 @@ def load():
     lib.dgo_visible_pairs.restype = C.c_uint64
     lib.dgo_attention_f32.argtypes = [P(Desc), VP, VP, VP, VP, VP, C.c_uint32, C.c_int]
     lib.dgo_attention_f64.argtypes = [P(Desc), VP, VP, VP, VP, VP, C.c_uint32, C.c_int]
+    lib.dgo_attention_topk_f32.argtypes = [P(Desc), P(C.c_uint32), VP, VP, VP, VP, C.c_uint32, VP, VP, C.c_uint32, C.c_int]
+    lib.dgo_topk_row_k.argtypes = [P(C.c_uint32), C.c_uint32, C.c_int]
+    lib.dgo_topk_row_k.restype = C.c_uint32
     lib.dgo_attention_blocked_f32.argtypes = [P(Desc), VP, VP, VP, VP, C.c_uint32, C.c_int]
     lib.dgo_attention_partial_f32.argtypes = [P(Desc), VP, VP, C.c_uint32, C.c_uint32, VP, VP, VP, C.c_int]
     lib.dgo_merge_partials_f32.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, VP, VP, VP, VP, VP]
@@ -127,6 +130,29 @@ def attention_f32(desc, q, kv, tok_list=None, n_threads=0):
     t, n = _toks(tok_list)
     load().dgo_attention_f32(C.byref(desc), _ptr(q), _ptr(kv), _ptr(out), _ptr(lse), _ptr(t), n, n_threads)
     return out, lse
+
+
+def topk_row_k(k_cfg, n_valid: int, causal_row: bool) -> int:
+    cfg = (C.c_uint32 * 4)(*k_cfg)
+    return int(load().dgo_topk_row_k(cfg, n_valid, 1 if causal_row else 0))
+
+
+def attention_topk_f32(desc, k_cfg, q, kv, tok_list=None, sel_cap=0, n_threads=0):
+    """Top-k sparse attention.  Returns out [canvas,Hq,hd] f32, or (out, sel_idx [canvas,Hq,sel_cap],
+    sel_count [canvas,Hq]) when sel_cap > 0."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    kv = np.ascontiguousarray(kv, dtype=np.float32)
+    out = np.zeros((desc.canvas, desc.n_q_heads, desc.head_dim), dtype=np.float32)
+    cfg = (C.c_uint32 * 4)(*k_cfg)
+    t, n = _toks(tok_list)
+    if sel_cap > 0:
+        idx = np.full((desc.canvas, desc.n_q_heads, sel_cap), 0xFFFFFFFF, dtype=np.uint32)
+        cnt = np.zeros((desc.canvas, desc.n_q_heads), dtype=np.uint32)
+        load().dgo_attention_topk_f32(C.byref(desc), cfg, _ptr(q), _ptr(kv), _ptr(out), _ptr(idx), sel_cap, _ptr(cnt),
+                                      _ptr(t), n, n_threads)
+        return out, idx, cnt
+    load().dgo_attention_topk_f32(C.byref(desc), cfg, _ptr(q), _ptr(kv), _ptr(out), None, 0, None, _ptr(t), n, n_threads)
+    return out
 
 
 def attention_f64(desc, q, kv, tok_list=None, n_threads=0):

@@ -64,6 +64,10 @@ def test_descriptor_validation_codes():
     assert _status(A.make_desc(256, 16, 2, 512, 1024, causal_rows=257)) == capi.DG_ERR_MASK
     assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_ring_mask=1000)) == capi.DG_ERR_LAYOUT
     assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_ring_mask=15)) == capi.DG_ERR_LAYOUT  # ring < key tile
+    # the ring must hold every visible position: window-1 + canvas of them
+    assert _status(A.make_desc(1024, 16, 8, 256, 4096, causal_rows=1024, window=1024, kv_ring_mask=2047)) == capi.DG_OK
+    assert _status(A.make_desc(1024, 16, 8, 256, 4096, causal_rows=1024, window=1026, kv_ring_mask=2047)) == capi.DG_ERR_LAYOUT
+    assert _status(A.make_desc(256, 16, 8, 256, 4096, kv_ring_mask=2047)) == capi.DG_ERR_LAYOUT  # no window: 4352 positions
     assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_dtype=7)) == capi.DG_ERR_DTYPE
     assert _status(A.make_desc(256, 16, 2, 512, 1024, q_dtype=capi.DG_F16, kv_dtype=capi.DG_BF16)) == capi.DG_ERR_DTYPE
     assert _status(A.make_desc(256, 16, 2, 512, 1024, out_dtype=capi.DG_F16)) == capi.DG_ERR_DTYPE
