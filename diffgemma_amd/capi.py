@@ -27,6 +27,8 @@ EXPORTS = (
     "dg_attn_visible_pairs", "dg_attention_dispatch", "dg_attention_state_bytes", "dg_kv_row_bytes",
     "dg_kv_region_bytes", "dg_kv_slot", "dg_layer_kv_slots", "dg_prof_begin", "dg_prof_end",
     "dg_calib_copy", "dg_calib_mfma", "dg_qk_rope_kv", "dg_qk_rope_kv_dispatch",
+    "dg_attn_topk_workspace_bytes", "dg_attn_topk_forward", "dg_attention_topk_state_bytes",
+    "dg_attention_topk_dispatch",
 )
 
 
@@ -145,6 +147,16 @@ def load():
     lib.dg_qk_rope_kv.restype = C.c_int
     lib.dg_qk_rope_kv_dispatch.argtypes = [VP, VP, VP, VP, VP, P(LayerOffsets), P(StepParams), P(AttnDims), VP, VP]
     lib.dg_qk_rope_kv_dispatch.restype = C.c_int
+    lib.dg_attn_topk_workspace_bytes.argtypes = [P(AttnDesc), P(C.c_uint32), P(C.c_size_t)]
+    lib.dg_attn_topk_workspace_bytes.restype = C.c_int
+    lib.dg_attn_topk_forward.argtypes = [P(AttnDesc), P(C.c_uint32), VP, VP, VP, VP, C.c_size_t, VP]
+    lib.dg_attn_topk_forward.restype = C.c_int
+    lib.dg_attention_topk_state_bytes.argtypes = [P(LayerOffsets), P(AttnDims), C.c_uint32, P(C.c_uint32),
+                                                  P(C.c_size_t)]
+    lib.dg_attention_topk_state_bytes.restype = C.c_int
+    lib.dg_attention_topk_dispatch.argtypes = [VP, VP, VP, P(LayerOffsets), P(StepParams), P(AttnDims),
+                                               P(C.c_uint32), VP, VP, C.c_size_t, VP]
+    lib.dg_attention_topk_dispatch.restype = C.c_int
     lib.dg_prof_begin.argtypes = [C.c_uint32]
     lib.dg_prof_begin.restype = C.c_int
     lib.dg_prof_end.argtypes = [P(C.c_double), P(C.c_uint32)]

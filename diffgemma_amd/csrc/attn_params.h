@@ -41,6 +41,20 @@ struct AttnParams {
   float scale_log2;      // softmax_scale * log2(e)
 };
 
+// One pass of top-k sparse attention over canvas rows [tok0, tok0 + ntok).
+constexpr int kTopkMaxK = 1024;   // most keys a row may keep
+struct TopkParams {
+  AttnParams a;          // tensors, strides and mask constants of the whole call
+  float* s_plane;        // scores [hq][ntok][t_pad], fp32
+  uint32_t tok0, ntok;
+  uint32_t t_pad;        // floats per score row, a multiple of the key tile
+  uint32_t n_mtiles;     // 128-row tiles of stacked rows in this pass
+  uint32_t n_splits;     // key-range splits of the score kernel (no merge needed)
+  uint32_t tile_first, tile_end;
+  uint32_t k_cfg[4];     // (fixed k | chunk grid, divisor, k_min, k_max)
+  float scale;
+};
+
 struct RowBounds {
   uint32_t lo, hi, extra;  // visible iff (lo <= t < hi) or (extra <= t), and t < t_all
 };
@@ -103,6 +117,8 @@ hipError_t launch_convert(const void* src, uint32_t src_dtype, void* dst, uint32
 hipError_t launch_kv_gather(const void* src, uint32_t src_dtype, void* dst, uint32_t dst_dtype, uint32_t hkv,
                             uint32_t t_all, uint32_t head_dim, int64_t tok_stride, int64_t head_stride,
                             uint32_t ring_mask, hipStream_t s);
+
+hipError_t launch_attn_topk(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 
 hipError_t launch_calib_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
 hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, hipStream_t s);

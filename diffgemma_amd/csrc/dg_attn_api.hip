@@ -261,24 +261,14 @@ int dg_attn_visible_pairs(const dg_attn_desc* d, uint64_t* pairs, double* flops)
   return DG_OK;
 }
 
-int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
-                    void* workspace, size_t workspace_bytes, void* stream) {
-  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
-  DeviceInfo di;
-  int rc = device_info(&di);
-  if (rc != DG_OK) return rc;
-  Plan pl;
-  rc = make_plan(d, 256, &pl);
-  if (rc != DG_OK) return rc;
-  if (pl.total > 0 && (!workspace || workspace_bytes < pl.total)) return DG_ERR_WORKSPACE;
-  if (pl.total > 0 && ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
-  if (((uintptr_t)q % 16) != 0 || ((uintptr_t)kv_base % 16) != 0 || ((uintptr_t)out % 16) != 0) return DG_ERR_LAYOUT;
-  hipStream_t s = (hipStream_t)stream;
-  char* ws = (char*)workspace;
+namespace {
+// Fills the kernel parameter block from a validated descriptor; runs the f32 -> f16 conversion
+// passes into the workspace when the plan asks for them.
+int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void* kv_base, void* out, float* lse,
+                char* ws, hipStream_t s, dg::AttnParams* pp) {
   const uint32_t hd = d->head_dim;
   const uint32_t esz_kv = elem_size(d->kv_dtype);
-
-  dg::AttnParams p;
+  dg::AttnParams& p = *pp;
   std::memset(&p, 0, sizeof(p));
   const char* region = (const char*)kv_base + d->kv_region_bytes;
   p.q = q;
@@ -334,6 +324,30 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
   p.out_dtype = d->out_dtype;
   p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
   p.scale_log2 = pl.scale * dg::kLog2e;
+  return DG_OK;
+}
+
+}  // namespace
+
+int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  if (pl.total > 0 && (!workspace || workspace_bytes < pl.total)) return DG_ERR_WORKSPACE;
+  if (pl.total > 0 && ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
+  if (((uintptr_t)q % 16) != 0 || ((uintptr_t)kv_base % 16) != 0 || ((uintptr_t)out % 16) != 0) return DG_ERR_LAYOUT;
+  hipStream_t s = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  const uint32_t hd = d->head_dim;
+
+  dg::AttnParams p;
+  rc = fill_params(d, pl, q, kv_base, out, lse, ws, s, &p);
+  if (rc != DG_OK) return rc;
   if (pl.n_splits > 1) {
     p.part_o = (float*)(ws + pl.off_part_o);
     p.part_ml = (float*)(ws + pl.off_part_ml);
@@ -355,6 +369,89 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
     ++g_prof.used;
   }
   if (pl.n_splits > 1 && dg::launch_attn_merge(p, hd, s) != hipSuccess) return DG_ERR_LAUNCH;
+  return DG_OK;
+}
+
+namespace {
+// Top-k sparse attention walks the canvas in row blocks so that the fp32 score plane of a block
+// ([Hq][rows][t_pad]) stays within the memory-side cache between the kernel that writes it and
+// the one that reads it.
+constexpr size_t kTopkPlaneBudget = 144ull << 20;
+
+struct TopkPlan {
+  uint32_t t_pad = 0, block_tok = 0;
+  size_t total = 0;
+};
+
+int make_topk_plan(const dg_attn_desc* d, const uint32_t* k_cfg, const Plan& pl, TopkPlan* tk) {
+  if (!k_cfg) return DG_ERR_NULL;
+  if (pl.scalar || d->q_dtype == DG_F32 || d->kv_dtype == DG_F32) return DG_ERR_UNSUPPORTED;
+  if (k_cfg[1] == 0u) {
+    if (k_cfg[0] > (uint32_t)dg::kTopkMaxK) return DG_ERR_SHAPE;
+  } else if (k_cfg[3] > (uint32_t)dg::kTopkMaxK || k_cfg[2] > k_cfg[3]) {
+    return DG_ERR_SHAPE;
+  }
+  tk->t_pad = (pl.t_all + dg::kBlockN - 1) / dg::kBlockN * dg::kBlockN;
+  const size_t per_tok = (size_t)d->n_q_heads * tk->t_pad * sizeof(float);
+  size_t blk = std::max<size_t>(1, kTopkPlaneBudget / per_tok);
+  if (blk >= 16) blk &= ~(size_t)15;
+  tk->block_tok = (uint32_t)std::min<size_t>(blk, d->canvas);
+  tk->total = align_up((size_t)tk->block_tok * per_tok);
+  return DG_OK;
+}
+}  // namespace
+
+int dg_attn_topk_workspace_bytes(const dg_attn_desc* d, const uint32_t* k_cfg, size_t* out_bytes) {
+  if (!d || !out_bytes) return DG_ERR_NULL;
+  Plan pl;
+  int rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  TopkPlan tk;
+  rc = make_topk_plan(d, k_cfg, pl, &tk);
+  if (rc != DG_OK) return rc;
+  *out_bytes = tk.total;
+  return DG_OK;
+}
+
+int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const void* q, const void* kv_base,
+                         void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, 256, &pl);
+  if (rc != DG_OK) return rc;
+  TopkPlan tk;
+  rc = make_topk_plan(d, k_cfg, pl, &tk);
+  if (rc != DG_OK) return rc;
+  if (!workspace || workspace_bytes < tk.total || ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
+  if (((uintptr_t)q % 16) != 0 || ((uintptr_t)kv_base % 16) != 0 || ((uintptr_t)out % 16) != 0) return DG_ERR_LAYOUT;
+  hipStream_t s = (hipStream_t)stream;
+
+  dg::TopkParams tp;
+  std::memset(&tp, 0, sizeof(tp));
+  rc = fill_params(d, pl, q, kv_base, out, nullptr, nullptr, s, &tp.a);   // no conversion passes: dtypes checked above
+  if (rc != DG_OK) return rc;
+  tp.a.dbg = g_tls_dbg;
+  tp.s_plane = (float*)workspace;
+  tp.t_pad = tk.t_pad;
+  tp.tile_first = pl.tile_first;
+  tp.tile_end = pl.tile_end;
+  for (int i = 0; i < 4; ++i) tp.k_cfg[i] = k_cfg[i];
+  tp.scale = pl.scale;
+  const uint32_t ntiles = std::max(1u, pl.tile_end - pl.tile_first);
+  for (uint32_t tok0 = 0; tok0 < d->canvas; tok0 += tk.block_tok) {
+    tp.tok0 = tok0;
+    tp.ntok = std::min(tk.block_tok, d->canvas - tok0);
+    tp.n_mtiles = (tp.ntok * pl.group + dg::kBlockM - 1) / dg::kBlockM;
+    // enough workgroups for every CU, no split shorter than 8 key tiles; splits write disjoint
+    // columns of the score plane, so there is nothing to merge
+    const uint32_t base = d->n_kv_heads * tp.n_mtiles;
+    uint32_t splits = std::max(1u, (256u + base - 1u) / base);
+    tp.n_splits = std::max(1u, std::min(splits, ntiles / 8u));
+    if (dg::launch_attn_topk(tp, d->head_dim, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+  }
   return DG_OK;
 }
 
@@ -393,6 +490,26 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
   desc_from_reference(L, dims, P->kv_len, &d);
   g_tls_dbg = (uint32_t*)dbg;
   const int rc = dg_attn_forward(&d, q, kvcache, out, nullptr, attn_state, attn_state_bytes, stream);
+  g_tls_dbg = nullptr;
+  return rc;
+}
+
+int dg_attention_topk_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                                  const uint32_t* k_cfg, size_t* out_bytes) {
+  if (!L || !dims || !out_bytes) return DG_ERR_NULL;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, kv_len, &d);
+  return dg_attn_topk_workspace_bytes(&d, k_cfg, out_bytes);
+}
+
+int dg_attention_topk_dispatch(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                               const dg_step_params* P, const dg_attn_dims* dims, const uint32_t* k_cfg,
+                               dg_debug_status* dbg, void* scratch, size_t scratch_bytes, void* stream) {
+  if (!L || !P || !dims) return DG_ERR_NULL;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, P->kv_len, &d);
+  g_tls_dbg = (uint32_t*)dbg;
+  const int rc = dg_attn_topk_forward(&d, k_cfg, q, kvcache, out, scratch, scratch_bytes, stream);
   g_tls_dbg = nullptr;
   return rc;
 }

@@ -159,6 +159,35 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
 int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
                              size_t* out_bytes);
 
+/* ---- top-k sparse attention (full-attention layers; the reference's default for them at depth) ----
+ *
+ * Replaces the three Metal kernels attn_gemm_qk (with the u16 key plane) + attn_topk_softmax +
+ * attn_topk_pv (src/shaders/attn/attention_topk/attention_topk.metal; encoded by
+ * StepEnc::encode_attn_decomp, src/metal/step_kernel/enc.rs:1820-2100) and their CPU twin
+ * (attention_topk/cpu.rs:41-120).  Per (query row, head): scores over the visible keys, the k
+ * highest kept (exact by fp32 score; equal scores: lower key position first, the CPU twin's
+ * rule), softmax over the kept keys only, their V rows summed.  Same descriptor, tensors, masks
+ * and layouts as dg_attn_forward; Q and the cache must be bf16 or f16 (no f32 inputs), LSE is
+ * not produced.
+ *
+ * k_cfg = the reference's (fixed_k | chunk grid, dyn_divisor, k_min, k_max)
+ * (src/flags/accessors.rs:210-221, attention_topk.metal:160-182): divisor 0 keeps k_cfg[0] keys
+ * (at least 1); otherwise a row keeps clamp(t_equiv / divisor, k_min, k_max) keys, t_equiv being
+ * its number of visible keys, rounded up to the grid for causal rows.  Never more than the row
+ * sees, never more than 1024. */
+int dg_attn_topk_workspace_bytes(const dg_attn_desc* d, const uint32_t* k_cfg, size_t* out_bytes);
+int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const void* q, const void* kv_base,
+                         void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same with the reference's argument block (bf16 Q/out with the truncating store, f16 cache at
+ * L->kv_region); `scratch` stands for the S / P / Idx / pattern planes the reference allocates
+ * (attention_topk/mod.rs:121-128), sized by dg_attention_topk_state_bytes. */
+int dg_attention_topk_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                                  const uint32_t* k_cfg, size_t* out_bytes);
+int dg_attention_topk_dispatch(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                               const dg_step_params* P, const dg_attn_dims* dims, const uint32_t* k_cfg,
+                               dg_debug_status* dbg, void* scratch, size_t scratch_bytes, void* stream);
+
 /* ---- the producer of the rows attention reads: per-head RMSNorm + RoPE + KV-cache write ----
  * Replaces the reference's qk_rope_kv kernel (src/shaders/attn/qk_rope_kv/qk_rope_kv.metal:29-149,
  * encoded by StepEnc::encode_layer_qk_rope_kv, src/metal/step_kernel/enc.rs:1739-1804; CPU twin
