@@ -262,6 +262,100 @@ def bench_schedule(args):
         sys.exit(1)
 
 
+TOPK_SHAPES = {   # canvas, Hq, Hkv, hd, kv_len, causal_rows: global layers of the stack
+    "topk_global": (256, 16, 2, 512, 32768, 0),              # denoise arm (causal = 0), k = t / 128 = 258
+    "topk_prefill_super": (1024, 16, 2, 512, 32768, 1024),   # prefill super-chunk, per-row k
+}
+
+
+def bench_topk(args):
+    """Top-k sparse attention of a global layer with the production k rule: one step = one
+    dg_attn_topk_forward (score kernel + select kernel per block of canvas rows)."""
+    import torch
+    from diffgemma_amd import attention as A, attention_topk as T, capi, rounding as R, workloads as W
+    from oracle import pyoracle as po
+    canvas, nq, nkv, hd, kv_len, cr = TOPK_SHAPES[args.workload]
+    w = W.Workload(args.workload, canvas, nq, nkv, hd, kv_len, causal_rows=cr, seed=41)
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+    d = w.desc()
+    k_cfg = T.adaptive_k()
+    ws = T.alloc_workspace(d, k_cfg)
+    out = torch.zeros(canvas * nq * hd, dtype=torch.int16, device="cuda")
+    pairs, _ = capi.visible_pairs(d)
+
+    T.forward(d, k_cfg, qd, kd, out, ws)
+    torch.cuda.synchronize()
+    od = po.make_desc(canvas, nq, nkv, hd, kv_len, causal_rows=cr, layout=w.layout, t_cap=w.t_all)
+    toks = np.unique(np.linspace(0, canvas - 1, max(2, args.check_toks)).round().astype(np.uint32))
+    t0 = time.perf_counter()
+    ref, idx, cnt = po.attention_topk_f32(od, k_cfg, q, kv, tok_list=toks, sel_cap=512)
+    t_cpu = time.perf_counter() - t0
+    got = R.bf16_bits_to_f32(out.cpu().numpy().view(np.uint16)).reshape(canvas, nq, hd)
+    diff = np.abs(got[toks] - ref[toks])
+    check = {"rows": int(len(toks)), "max_abs": float(diff.max()), "mean_abs": float(diff.mean()),
+             "keys_kept_min_max": [int(cnt[toks].min()), int(cnt[toks].max())],
+             "tol": {"max_abs": 2e-2, "mean_abs": 2e-3}}
+    check["passed"] = bool(diff.max() <= 2e-2 and diff.mean() <= 2e-3 and np.isfinite(got).all())
+
+    for _ in range(args.warmup):
+        T.forward(d, k_cfg, qd, kd, out, ws)
+    torch.cuda.synchronize()
+    n_blocks = -(-canvas // max(1, (T.workspace_bytes(d, k_cfg) // (nq * 4 * (-(-w.t_all // 32) * 32)))))
+    capi.prof_begin(2 * n_blocks * args.steps + 2)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        T.forward(d, k_cfg, qd, kd, out, ws)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    scores_ms, select_ms, n_pairs = capi.prof_end_split()
+    scores_ms /= args.steps
+    select_ms /= args.steps
+    ms = (t1 - t0) * 1e3 / args.steps
+
+    # algorithmic work: the score kernel multiplies every visible (row, key) pair once (2 * hd flop);
+    # the select kernel reads every visible fp32 score once, gathers the kept V rows and writes the row
+    kept = float(sum(min(max((-(-(kv_len + t + 1) // 256) * 256 if t < cr else w.t_all) // 128, 64), 512)
+                     for t in range(canvas)))
+    qk_flops = 2.0 * hd * nq * pairs
+    # (the gathered V rows of a block of canvas rows come from at most the whole V plane: what is
+    # gathered beyond that is cache traffic, reported separately)
+    gathered = kept * nq * hd * 2
+    row_blocks = -(-canvas // max(1, (T.workspace_bytes(d, k_cfg) // (nq * 4 * (-(-w.t_all // 32) * 32)))))
+    sel_bytes = 4.0 * nq * pairs + min(gathered, row_blocks * float(w.t_all * nkv * hd * 2)) + canvas * nq * hd * 2
+    score_bytes = 4.0 * nq * pairs + w.t_all * nkv * hd * 2 + canvas * nq * hd * 2
+    dominant_is_select = select_ms >= scores_ms
+    roof = ({"bound": "hbm", "achieved": sel_bytes / (select_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+             "kernel": "topk_select_kernel", "kernel_ms": select_ms} if dominant_is_select else
+            {"bound": "mfma", "achieved": qk_flops / (scores_ms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+             "unit": "TFLOP/s", "kernel": "topk_scores_kernel", "kernel_ms": scores_ms})
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    res = {"metric": f"top-k sparse attention of a global layer ({canvas}-row canvas @ {kv_len} prefix, k = t/128): "
+                     "canvas tokens/s, 1 GPU",
+           "value": canvas / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+           "data": "synthetic",
+           "config": {"workload": args.workload, "canvas": canvas, "kv_prefix": kv_len, "n_q_heads": nq, "n_kv_heads": nkv,
+                      "head_dim": hd, "causal_rows": cr, "k_cfg": list(k_cfg), "row_blocks": n_blocks,
+                      "score_plane_bytes": T.workspace_bytes(d, k_cfg)},
+           "kernels": {"topk_scores_kernel": {"ms": scores_ms, "tflops": qk_flops / (scores_ms * 1e-3) / 1e12,
+                                              "frac_mfma_peak": qk_flops / (scores_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                              "written_gbs": 4.0 * nq * pairs / (scores_ms * 1e-3) / 1e9,
+                                              "algorithmic_bytes": score_bytes},
+                       "topk_select_kernel": {"ms": select_ms, "gbs": sel_bytes / (select_ms * 1e-3) / 1e9,
+                                              "algorithmic_bytes": sel_bytes, "gathered_v_bytes": gathered}},
+           "roofline": roof, "check": check}
+    if not args.no_cpu_baseline:
+        threads = min(po.max_threads(), 16)
+        res["cpu_baseline"] = {"value": len(toks) / t_cpu, "unit": "tokens/s", "cores": threads, "kind": "port",
+                               "sample": f"{len(toks)} of {canvas} canvas rows x all {nq} heads, {t_cpu:.2f} s, port of the "
+                                         "reference's CPU top-k attention (full sort replaced by a partial sort), OpenMP"}
+    print(json.dumps(res), flush=True)
+    if not check["passed"]:
+        sys.exit(1)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -292,6 +386,9 @@ def main():
         return
     if args.workload == "cfg5_schedule":
         bench_schedule(args)
+        return
+    if args.workload in TOPK_SHAPES:
+        bench_topk(args)
         return
 
     w = W.config(args.workload)

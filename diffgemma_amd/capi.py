@@ -28,7 +28,7 @@ EXPORTS = (
     "dg_kv_region_bytes", "dg_kv_slot", "dg_layer_kv_slots", "dg_prof_begin", "dg_prof_end",
     "dg_calib_copy", "dg_calib_mfma", "dg_qk_rope_kv", "dg_qk_rope_kv_dispatch",
     "dg_attn_topk_workspace_bytes", "dg_attn_topk_forward", "dg_attention_topk_state_bytes",
-    "dg_attention_topk_dispatch",
+    "dg_attention_topk_dispatch", "dg_prof_end_split",
 )
 
 
@@ -161,6 +161,8 @@ def load():
     lib.dg_prof_begin.restype = C.c_int
     lib.dg_prof_end.argtypes = [P(C.c_double), P(C.c_uint32)]
     lib.dg_prof_end.restype = C.c_int
+    lib.dg_prof_end_split.argtypes = [P(C.c_double), P(C.c_double), P(C.c_uint32)]
+    lib.dg_prof_end_split.restype = C.c_int
     _lib = lib
     return lib
 
@@ -194,6 +196,13 @@ def visible_pairs(desc: AttnDesc):
 
 def prof_begin(max_launches: int) -> None:
     check(load().dg_prof_begin(max_launches))
+
+
+def prof_end_split():
+    """Returns (ms of even-numbered event pairs, ms of odd-numbered ones, pairs recorded)."""
+    a, b, n = C.c_double(0.0), C.c_double(0.0), C.c_uint32(0)
+    check(load().dg_prof_end_split(C.byref(a), C.byref(b), C.byref(n)))
+    return a.value, b.value, n.value
 
 
 def prof_end():

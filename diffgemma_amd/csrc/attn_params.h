@@ -118,7 +118,8 @@ hipError_t launch_kv_gather(const void* src, uint32_t src_dtype, void* dst, uint
                             uint32_t t_all, uint32_t head_dim, int64_t tok_stride, int64_t head_stride,
                             uint32_t ring_mask, hipStream_t s);
 
-hipError_t launch_attn_topk(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
+hipError_t launch_topk_scores(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
+hipError_t launch_topk_select(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 
 hipError_t launch_calib_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
 hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, hipStream_t s);

@@ -24,7 +24,22 @@
 namespace dg {
 namespace {
 
-constexpr int kCandCap = 4096;     // LDS candidate list of the select kernel
+constexpr int kCandCap = 2048;     // LDS candidate list of the select kernel (sized for 4 workgroups per CU)
+
+// Optional per-phase cycle accounting of the select kernel (development builds only): thread 0 of
+// every workgroup adds the cycles it spent in each phase to eight global sums.
+#ifdef DG_ATTN_PHASE_TIMING
+#define TK_PHASE_DECL unsigned long long tk_t = clock64();
+#define TK_PHASE(i)                                                        \
+  if (p.phase_cycles && tid == 0) {                                        \
+    const unsigned long long now = clock64();                              \
+    atomicAdd(&p.phase_cycles[i], now - tk_t);                             \
+    tk_t = now;                                                            \
+  }
+#else
+#define TK_PHASE_DECL
+#define TK_PHASE(i)
+#endif
 // radix digits of the 32-bit key, most significant first: 11 + 11 + 10 bits
 __device__ __forceinline__ uint32_t digit_shift(int level) { return level == 0 ? 21u : level == 1 ? 10u : 0u; }
 __device__ __forceinline__ uint32_t digit_bits(int level) { return level == 2 ? 10u : 11u; }
@@ -101,7 +116,7 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
   const uint32_t te = __builtin_amdgcn_readfirstlane(min(tb + per_split, mt_end));
   if (te <= tb) return;
 
-  // Q fragments: B operand of S^T = K.Q^T, lane = row, 8 consecutive d per step
+  // Q fragments: lane = row, 8 consecutive d per step
   u32x4 qf[NSTEP];
   {
     const size_t qoff = ((size_t)tok * p.hq + qh) * D + 8u * g2;
@@ -127,46 +142,95 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
   const uint32_t t_last = (te - 1u) * kBlockN;
   // loads for a tile past the last one fetch the last tile again into a buffer nobody reads, so
   // that every iteration issues the same number of loads and the wait counts stay fixed
-  auto issue_k = [&](uint32_t j) {
+  auto k_desc = [&](uint32_t j) {
     lds_char* buf = (lds_char*)(smem + ((j - tb) % NB) * L::K_BYTES);
-    const TileLoad tl = make_tile_load<D, false, false>(kbase, kstride_b, min(j * kBlockN, t_last), 0u, p.t_all,
-                                                        p.ring_mask, buf, wave, lane);
-    issue_tile<D, false>(tl, wave, lane);
+    return make_tile_load<D, false, false>(kbase, kstride_b, min(j * kBlockN, t_last), 0u, p.t_all, p.ring_mask, buf,
+                                           wave, lane);
   };
-  float* const srow = tp.s_plane + ((size_t)qh * tp.ntok + tok_l) * tp.t_pad;
+  auto issue_k = [&](uint32_t j) { issue_tile<D, false>(k_desc(j), wave, lane); };
+  // The product is taken as S = Q.K^T (A = Q, B = K): the output lane is then the key and
+  // register e of the block is query row 8 (e >> 2) + 4 g2 + (e & 3) of this wave's 32, so one
+  // store instruction writes 32 consecutive keys of two rows: whole 128-byte lines.  (With the
+  // operands the other way round every store scatters 32-byte pieces over 32 rows and the
+  // kernel is bound by the write path.)  Where each of the 16 rows lives, and whether it exists:
+  uint32_t row_off[16];      // float offset of the row in the score plane, without the key
+  uint32_t row_mask = 0;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const uint32_t rr = row0 + wave * 32u + 8u * (e >> 2) + 4u * g2 + (e & 3);
+    const bool ok = rr < rows_total;
+    const uint32_t tl = ok ? rr / p.group : 0u;
+    const uint32_t hh = kvh * p.group + (ok ? rr % p.group : 0u);
+    row_off[e] = (hh * tp.ntok + tl) * tp.t_pad;
+    row_mask |= ok ? 1u << e : 0u;
+  }
 
 #pragma unroll
   for (int i = 0; i < PF; ++i) issue_k(tb + i);
+  // lane l32 holds key t0 + l32 of sixteen rows
+  auto store_tile = [&](const f32x16& sc, uint32_t tile) {
+    float* const dst = tp.s_plane + tile * kBlockN + l32;
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      if (row_mask & (1u << e)) dst[row_off[e]] = sc[e] * tp.scale;
+  };
+  f32x16 s_prev;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) s_prev[e] = 0.f;
   for (uint32_t j = tb; j < te; ++j) {
     // this wave's loads of K(j) have landed (the PF-1 tiles behind it may still be in flight);
     // after the barrier everybody's have, and everybody is done reading K(j-1), whose buffer
-    // takes K(j+PF)
+    // takes K(j+PF).  The scores of tile j-1 are stored only now, a tile late: stores count in
+    // the same counter as the loads, and issued right before the wait they would have to drain
+    // first; issued here they are a tile old at the next wait.
     wait_loads_then_barrier<(PF - 1) * NLD>();
-    issue_k(j + PF);
+    if (j > tb) store_tile(s_prev, j - 1u);
+    // (the loads of K(j+PF) are issued between the MFMAs below: back to back each of them holds
+    // the wave's issue slot for about two MFMAs' worth of cycles)
+    const TileLoad tl_next = k_desc(j + PF);
     lds_char* const kb = (lds_char*)(smem + ((j - tb) % NB) * L::K_BYTES);
     f32x16 s;
 #pragma unroll
     for (int e = 0; e < 16; ++e) s[e] = 0.f;
+    // K fragments in chunks of CH: the reads of chunk c+1 are issued before the MFMAs of chunk c
+    // (left to itself the compiler reads two fragments, waits, multiplies, and the LDS latency
+    // is paid sixteen times per tile)
+    constexpr int CH = NSTEP < 8 ? NSTEP : 8;
+    constexpr int NCHUNK = NSTEP / CH;
+    constexpr int LPC = (NLD + NCHUNK - 1) / NCHUNK;      // tile loads issued per chunk
+    constexpr int LGAP = CH / LPC;                         // MFMAs between two of them
+    static_assert(LPC * NCHUNK >= NLD && LPC <= CH, "tile loads must fit between the MFMAs");
+    u32x4 fr[2][CH];
+    auto read_chunk = [&](int c, u32x4 (&dst)[CH]) {
 #pragma unroll
-    for (int st = 0; st < NSTEP; ++st) {
-      u32x4 a;
-      if constexpr (L::PAD) {
-        a = *(lds_u32x4*)(kb + k_lane_off + 32 * st);
-      } else {
-        const uint32_t c = (uint32_t)(2 * st) + g2;
-        a = *(lds_u32x4*)(kb + k_lane_off + ((c ^ k_swz) << 4));
+      for (int i = 0; i < CH; ++i) {
+        const int st = c * CH + i;
+        if constexpr (L::PAD) {
+          dst[i] = *(lds_u32x4*)(kb + k_lane_off + 32 * st);
+        } else {
+          const uint32_t cc = (uint32_t)(2 * st) + g2;
+          dst[i] = *(lds_u32x4*)(kb + k_lane_off + ((cc ^ k_swz) << 4));
+        }
       }
-      s = mfma16<F16>(a, qf[st], s);
-    }
-    // register e of the block is key t0 + 8 (e >> 2) + 4 g2 + (e & 3) of row l32
-    if (row_ok) {
-      float* dst = srow + j * kBlockN + 4u * g2;
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4)
-        *(f32x4*)(dst + 8 * q4) = f32x4{s[4 * q4] * tp.scale, s[4 * q4 + 1] * tp.scale, s[4 * q4 + 2] * tp.scale,
-                                         s[4 * q4 + 3] * tp.scale};
-    }
+    };
+    read_chunk(0, fr[0]);
+    static_for<0, NCHUNK>([&](auto c_c) {
+      constexpr int c = decltype(c_c)::value;
+      if constexpr (c + 1 < NCHUNK) read_chunk(c + 1, fr[(c + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<0, CH>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        s = mfma16<F16>(qf[c * CH + i], fr[c & 1][i], s);
+        if constexpr (i % LGAP == LGAP / 2 && c * LPC + i / LGAP < NLD) {
+          issue_tile_part<D, false, c * LPC + i / LGAP>(tl_next, wave, lane);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    s_prev = s;
   }
+  store_tile(s_prev, te - 1u);
   wait_vmem_all();   // no direct-to-LDS load may outlive the workgroup's LDS
 }
 
@@ -179,6 +243,11 @@ __device__ __forceinline__ uint32_t score_key(float f) {
   const uint32_t u = __float_as_uint(f);
   if ((u & 0x7fffffffu) > 0x7f800000u) return 0u;
   return (u & 0x80000000u) ? ~u : (u ^ 0x80000000u);
+}
+
+// the score a key stands for (inverse of score_key for every non-NaN score)
+__device__ __forceinline__ float key_score(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
 }
 
 // number of keys row bounds b let through
@@ -208,6 +277,7 @@ struct SelectShared {
 // threads call it; it contains barriers.
 __device__ __forceinline__ void pick_bin(SelectShared& sh, uint32_t nbins, uint32_t remaining, uint32_t tid) {
   const uint32_t per = nbins >> 8;          // bins per thread: 8 or 4
+  const uint32_t lane = tid & 63u, wave = tid >> 6;
   uint32_t c[8];
   uint32_t sum = 0;
 #pragma unroll
@@ -215,10 +285,18 @@ __device__ __forceinline__ void pick_bin(SelectShared& sh, uint32_t nbins, uint3
     c[i] = i < per ? sh.hist[tid * per + i] : 0u;
     sum += c[i];
   }
-  sh.tot[tid] = sum;
+  // entries in the bins of higher threads: suffix sum over the lanes of the wave, then the
+  // totals of the higher waves
+  uint32_t incl = sum;
+#pragma unroll
+  for (uint32_t off = 1; off < 64u; off <<= 1) {
+    const uint32_t v = __shfl_down(incl, off, 64);
+    if (lane + off < 64u) incl += v;
+  }
+  if (lane == 0) sh.tot[wave] = incl;
   __syncthreads();
-  uint32_t above = 0;                        // entries in the bins of higher threads
-  for (uint32_t t = tid + 1; t < 256u; ++t) above += sh.tot[t];
+  uint32_t above = incl - sum;
+  for (uint32_t w = wave + 1; w < 4u; ++w) above += sh.tot[w];
   if (above < remaining && remaining <= above + sum) {
     uint32_t run = above;
 #pragma unroll
@@ -234,6 +312,36 @@ __device__ __forceinline__ void pick_bin(SelectShared& sh, uint32_t nbins, uint3
     }
   }
   __syncthreads();
+}
+
+// The `need`-th largest of the keys key_of(i) yields for i in [0, n) (key_of returns false for
+// entries that do not take part), by three histogram levels over LDS.  Returns the key; *n_equal
+// = entries equal to it, *take_equal = how many of those belong to the `need` largest.  All 256
+// threads call it with the same arguments; needs 1 <= need <= number of participating entries.
+template <typename KeyOf>
+__device__ __forceinline__ uint32_t lds_kth_largest(SelectShared& sh, uint32_t n, uint32_t need, uint32_t tid,
+                                                    KeyOf&& key_of, uint32_t* take_equal, uint32_t* n_equal) {
+  uint32_t prefix = 0, pbits = 0, remaining = need, cls = 0;
+  for (int lv = 0; lv < 3; ++lv) {
+    const uint32_t nbins = 1u << digit_bits(lv);
+    for (uint32_t b = tid; b < nbins; b += 256u) sh.hist[b] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < n; i += 256u) {
+      uint32_t key;
+      if (key_of(i, key) && (pbits == 0u || (key >> (32u - pbits)) == prefix))
+        atomicAdd(&sh.hist[(key >> digit_shift(lv)) & (nbins - 1u)], 1u);
+    }
+    __syncthreads();
+    pick_bin(sh, nbins, remaining, tid);
+    remaining -= sh.res[1];
+    prefix = (prefix << digit_bits(lv)) | sh.res[0];
+    pbits += digit_bits(lv);
+    cls = sh.res[2];
+    __syncthreads();
+  }
+  *take_equal = remaining;
+  *n_equal = cls;
+  return prefix;
 }
 
 template <int D, bool F16>
@@ -275,31 +383,100 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
   const uint32_t hull_lo = (rb.extra < p.t_all ? min(rb.lo, rb.extra) : rb.lo) & ~3u;
   const uint32_t hull_hi = rb.extra < p.t_all ? p.t_all : min(rb.hi, p.t_all);
 
+  // f(position, score) for every visible key of the row; each thread takes one float4 out of
+  // every 256 and has four of them in flight
+  auto scan_row = [&](auto&& f) {
+    for (uint32_t t4 = hull_lo + 4u * tid; t4 < hull_hi; t4 += 4096u) {
+      f32x4 v[4];
+#pragma unroll
+      for (uint32_t u = 0; u < 4; ++u) {
+        const uint32_t a = t4 + 1024u * u;
+        v[u] = a < hull_hi ? *(const f32x4*)(srow + a) : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < 4; ++u) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+          const uint32_t t = t4 + 1024u * u + i;
+          if (t < hull_hi && key_visible(rb, t, p.t_all)) f(t, v[u][i]);
+        }
+      }
+    }
+  };
+
+  TK_PHASE_DECL
   if (tid == 0) {
     sh.n_sel = 0;
     sh.n_cand = 0;
     sh.res[0] = sh.res[1] = sh.res[2] = 0;
   }
 
-  // ---- levels over the score row in memory, until the class of the k-th score fits the list ----
   uint32_t prefix = 0, pbits = 0, remaining = k, class_count = n_valid;
   int level = 0;
-  for (; level < 3 && class_count > (uint32_t)kCandCap; ++level) {
+  bool have_cand = false;   // the candidate list already holds every key at or above a sampled threshold
+
+  // ---- long rows: cut at a threshold taken from a sample, so that the row is read once ----
+  // About 2048 keys at an even stride give the key tau below which ~2.5 k keys are expected;
+  // one pass collects everything >= tau.  If that is at least k and fits the list, the exact
+  // k-th key is found in LDS; otherwise (an unlucky or clustered sample) the exact histogram
+  // levels below run instead.
+  if (n_valid > (uint32_t)kCandCap) {
+    const uint32_t stride = max(1u, (hull_hi - hull_lo + 2047u) / 2048u);
+    const uint32_t m = (hull_hi - hull_lo + stride - 1u) / stride;     // sample slots, at most 2048
+    {
+      float sv[8];
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) {      // m <= 2048: eight samples per thread, all in flight
+        const uint32_t i = tid + 256u * u;
+        sv[u] = i < m ? srow[hull_lo + i * stride] : 0.f;
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) {
+        const uint32_t i = tid + 256u * u;
+        // (an invisible position takes part as the lowest key, which cannot reach the top ranks asked for)
+        if (i < m) sh.cand_key[i] = key_visible(rb, hull_lo + i * stride, p.t_all) ? score_key(sv[u]) : 0u;
+      }
+    }
+    __syncthreads();
+    if (m > 0u) {
+      // aim at ~2.5 k keys at or above tau, but never beyond 3/4 of the list
+      const uint64_t want = min<uint64_t>(5ull * k / 2ull, 3ull * kCandCap / 4ull);
+      const uint32_t r = min(m, (uint32_t)((want * m + n_valid - 1ull) / n_valid) + 8u);
+      uint32_t te, ne;
+      TK_PHASE(7)
+      const uint32_t tau = lds_kth_largest(
+          sh, m, r, tid, [&](uint32_t i, uint32_t& key) { key = sh.cand_key[i]; return true; }, &te, &ne);
+      TK_PHASE(1)
+      scan_row([&](uint32_t t, float sv) {
+        const uint32_t key = score_key(sv);
+        if (key >= tau) {
+          const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
+          if (slot < (uint32_t)kCandCap) {
+            sh.cand_key[slot] = key;
+            sh.cand_t[slot] = t;
+          }
+        }
+      });
+      __syncthreads();
+      const uint32_t got = sh.n_cand;
+      have_cand = got >= k && got <= (uint32_t)kCandCap;
+      if (have_cand) class_count = got;
+      __syncthreads();
+      if (!have_cand && tid == 0) sh.n_cand = 0;
+    }
+    __syncthreads();
+  }
+
+  // ---- exact levels over the score row in memory, until the class of the k-th score fits the list ----
+  for (; !have_cand && level < 3 && class_count > (uint32_t)kCandCap; ++level) {
     const uint32_t nbins = 1u << digit_bits(level);
     for (uint32_t b = tid; b < nbins; b += 256u) sh.hist[b] = 0;
     __syncthreads();
-    for (uint32_t t4 = hull_lo + 4u * tid; t4 < hull_hi; t4 += 1024u) {
-      const f32x4 v = *(const f32x4*)(srow + t4);
-#pragma unroll
-      for (uint32_t i = 0; i < 4; ++i) {
-        const uint32_t t = t4 + i;
-        if (key_visible(rb, t, p.t_all)) {
-          const uint32_t key = score_key(v[i]);
-          if (pbits == 0u || (key >> (32u - pbits)) == prefix)
-            atomicAdd(&sh.hist[(key >> digit_shift(level)) & (nbins - 1u)], 1u);
-        }
-      }
-    }
+    scan_row([&](uint32_t, float sv) {
+      const uint32_t key = score_key(sv);
+      if (pbits == 0u || (key >> (32u - pbits)) == prefix)
+        atomicAdd(&sh.hist[(key >> digit_shift(level)) & (nbins - 1u)], 1u);
+    });
     __syncthreads();
     pick_bin(sh, nbins, remaining, tid);
     remaining -= sh.res[1];
@@ -309,24 +486,20 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
     __syncthreads();
   }
 
+  TK_PHASE(0)
   if (class_count > (uint32_t)kCandCap) {
     // More than a list's worth of bit-identical scores at the threshold (a degenerate row, e.g.
     // an all-zero query).  Keys above go in as they come; of the ties the first `remaining` by
     // position are taken by one wave walking the row in order.
-    for (uint32_t t4 = hull_lo + 4u * tid; t4 < hull_hi; t4 += 1024u) {
-      const f32x4 v = *(const f32x4*)(srow + t4);
-#pragma unroll
-      for (uint32_t i = 0; i < 4; ++i) {
-        const uint32_t t = t4 + i;
-        if (key_visible(rb, t, p.t_all) && score_key(v[i]) > prefix) {
-          const uint32_t slot = atomicAdd(&sh.n_sel, 1u);
-          if (slot < (uint32_t)kTopkMaxK) {
-            sh.sel_s[slot] = v[i];
-            sh.sel_t[slot] = t;
-          }
+    scan_row([&](uint32_t t, float sv) {
+      if (score_key(sv) > prefix) {
+        const uint32_t slot = atomicAdd(&sh.n_sel, 1u);
+        if (slot < (uint32_t)kTopkMaxK) {
+          sh.sel_s[slot] = sv;
+          sh.sel_t[slot] = t;
         }
       }
-    }
+    });
     __syncthreads();
     if (wave == 0) {
       const uint32_t first = k - remaining;
@@ -350,85 +523,78 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
     }
     __syncthreads();
   } else {
-    // ---- one pass: keys above the class go straight to the kept list, the class to the candidates ----
-    for (uint32_t t4 = hull_lo + 4u * tid; t4 < hull_hi; t4 += 1024u) {
-      const f32x4 v = *(const f32x4*)(srow + t4);
-#pragma unroll
-      for (uint32_t i = 0; i < 4; ++i) {
-        const uint32_t t = t4 + i;
-        if (key_visible(rb, t, p.t_all)) {
-          const uint32_t key = score_key(v[i]);
-          const uint32_t hi = pbits ? key >> (32u - pbits) : 0u;
-          if (hi > prefix) {
-            const uint32_t slot = atomicAdd(&sh.n_sel, 1u);
-            if (slot < (uint32_t)kTopkMaxK) {
-              sh.sel_s[slot] = v[i];
-              sh.sel_t[slot] = t;
-            }
-          } else if (hi == prefix) {
-            const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
-            if (slot < (uint32_t)kCandCap) {
-              sh.cand_key[slot] = key;
-              sh.cand_t[slot] = t;
-            }
+    if (!have_cand) {
+      // ---- one pass: keys above the class go straight to the kept list, the class to the candidates ----
+      scan_row([&](uint32_t t, float sv) {
+        const uint32_t key = score_key(sv);
+        const uint32_t hi = pbits ? key >> (32u - pbits) : 0u;
+        if (hi > prefix) {
+          const uint32_t slot = atomicAdd(&sh.n_sel, 1u);
+          if (slot < (uint32_t)kTopkMaxK) {
+            sh.sel_s[slot] = sv;
+            sh.sel_t[slot] = t;
+          }
+        } else if (hi == prefix) {
+          const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
+          if (slot < (uint32_t)kCandCap) {
+            sh.cand_key[slot] = key;
+            sh.cand_t[slot] = t;
           }
         }
-      }
+      });
+      __syncthreads();
     }
-    __syncthreads();
+    TK_PHASE(1)
     const uint32_t n_cand = min(sh.n_cand, (uint32_t)kCandCap);
 
-    // ---- remaining levels over the candidate list ----
-    for (; level < 3; ++level) {
-      const uint32_t nbins = 1u << digit_bits(level);
-      for (uint32_t b = tid; b < nbins; b += 256u) sh.hist[b] = 0;
-      __syncthreads();
-      for (uint32_t i = tid; i < n_cand; i += 256u) {
-        const uint32_t key = sh.cand_key[i];
-        if (pbits == 0u || (key >> (32u - pbits)) == prefix)
-          atomicAdd(&sh.hist[(key >> digit_shift(level)) & (nbins - 1u)], 1u);
-      }
-      __syncthreads();
-      pick_bin(sh, nbins, remaining, tid);
-      remaining -= sh.res[1];
-      prefix = (prefix << digit_bits(level)) | sh.res[0];
-      pbits += digit_bits(level);
-      class_count = sh.res[2];
-      __syncthreads();
-    }
-    // prefix is now the k-th largest key; `remaining` of the class_count keys equal to it are kept
-
-    // ---- equal scores: the lower positions win.  Threshold on position by the same select ----
-    uint32_t t_key_min = 0u;   // ties with ~t >= t_key_min are kept
-    if (class_count > remaining) {
-      uint32_t tp_prefix = 0, tp_bits = 0, tp_rem = remaining;
-      for (int lv = 0; lv < 3; ++lv) {
+    // ---- the k-th key among the candidates: the levels not yet done, over the list ----
+    uint32_t thr = prefix, take_eq = remaining, n_eq = class_count;
+    if (level < 3) {
+      // (the list holds exactly the keys whose leading pbits bits equal prefix: rebuild the full
+      // key of the threshold from the remaining levels)
+      uint32_t lp = prefix, lb = pbits, rem = remaining, cls = class_count;
+      for (int lv = level; lv < 3; ++lv) {
         const uint32_t nbins = 1u << digit_bits(lv);
         for (uint32_t b = tid; b < nbins; b += 256u) sh.hist[b] = 0;
         __syncthreads();
         for (uint32_t i = tid; i < n_cand; i += 256u) {
-          if (sh.cand_key[i] == prefix) {
-            const uint32_t key2 = ~sh.cand_t[i];
-            if (tp_bits == 0u || (key2 >> (32u - tp_bits)) == tp_prefix)
-              atomicAdd(&sh.hist[(key2 >> digit_shift(lv)) & (nbins - 1u)], 1u);
-          }
+          const uint32_t key = sh.cand_key[i];
+          if (lb == 0u || (key >> (32u - lb)) == lp) atomicAdd(&sh.hist[(key >> digit_shift(lv)) & (nbins - 1u)], 1u);
         }
         __syncthreads();
-        pick_bin(sh, nbins, tp_rem, tid);
-        tp_rem -= sh.res[1];
-        tp_prefix = (tp_prefix << digit_bits(lv)) | sh.res[0];
-        tp_bits += digit_bits(lv);
+        pick_bin(sh, nbins, rem, tid);
+        rem -= sh.res[1];
+        lp = (lp << digit_bits(lv)) | sh.res[0];
+        lb += digit_bits(lv);
+        cls = sh.res[2];
         __syncthreads();
       }
-      t_key_min = tp_prefix;
+      thr = lp;
+      take_eq = rem;
+      n_eq = cls;
+    }
+    // thr is the k-th largest key; take_eq of the n_eq keys equal to it are kept
+    TK_PHASE(6)
+
+    // ---- equal scores: the lower positions win.  Threshold on position by the same select ----
+    uint32_t t_key_min = 0u;   // ties with ~t >= t_key_min are kept
+    if (n_eq > take_eq) {
+      uint32_t te, ne;
+      t_key_min = lds_kth_largest(
+          sh, n_cand, take_eq, tid,
+          [&](uint32_t i, uint32_t& key) {
+            key = ~sh.cand_t[i];
+            return sh.cand_key[i] == thr;
+          },
+          &te, &ne);
     }
     for (uint32_t i = tid; i < n_cand; i += 256u) {
       const uint32_t key = sh.cand_key[i];
       const uint32_t t = sh.cand_t[i];
-      if (key > prefix || (key == prefix && ~t >= t_key_min)) {
+      if (key > thr || (key == thr && ~t >= t_key_min)) {
         const uint32_t slot = atomicAdd(&sh.n_sel, 1u);
         if (slot < (uint32_t)kTopkMaxK) {
-          sh.sel_s[slot] = srow[t];
+          sh.sel_s[slot] = key_score(key);
           sh.sel_t[slot] = t;
         }
       }
@@ -436,6 +602,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
     __syncthreads();
   }
 
+  TK_PHASE(2)
   // ---- sort the kept keys by position (bitonic, padded with +inf positions) ----
   uint32_t npow = 1;
   while (npow < k) npow <<= 1;
@@ -463,6 +630,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
     }
   }
 
+  TK_PHASE(3)
   // ---- softmax over the kept scores (cpu.rs:95-104) ----
   float* const fred = (float*)sh.hist;   // histogram storage is free now
   float m = -INFINITY;
@@ -490,6 +658,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
   const float lsum = fred[0];
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
 
+  TK_PHASE(4)
   // ---- gathered P.V: wave w takes kept keys w, w+4, ...; a lane owns PER consecutive d ----
   constexpr int PER = D >= 64 ? D / 64 : 1;
   const bool lane_on = lane * PER < (uint32_t)D;
@@ -498,40 +667,55 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
   for (int i = 0; i < PER; ++i) acc[i] = 0.f;
   const char* vbase = (const char*)p.v + (int64_t)kvh * p.v_head_stride * 2 + (size_t)lane * PER * 2;
   const int64_t vstride_b = p.v_tok_stride * 2;
-  for (uint32_t j = wave; j < k; j += 4u) {
-    const float pj = sh.sel_s[j] * inv;
-    const uint32_t tj = min(sh.sel_t[j], p.t_all - 1u);   // (kept positions are < t_all by construction)
-    const uint16_t* vp = (const uint16_t*)(vbase + (int64_t)kv_slot(p.ring_mask, tj) * vstride_b);
-    if (lane_on) {
-      uint16_t raw[PER];
-      if constexpr (PER == 8) {
-        const u32x4 x = *(const u32x4*)vp;
+  // kept keys in groups of GU per wave (wave w takes groups w, w+4, ...): the GU row loads of a
+  // group are issued before any of them is used, so a row's latency is paid once per group
+  constexpr int GU = 8;
+  auto load_row = [&](const uint16_t* vp, uint16_t (&raw)[PER]) {
+    if constexpr (PER == 8) {
+      const u32x4 x = *(const u32x4*)vp;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          raw[2 * i] = (uint16_t)(x[i] & 0xffffu);
-          raw[2 * i + 1] = (uint16_t)(x[i] >> 16);
-        }
-      } else if constexpr (PER == 4) {
-        const u32x2 x = *(const u32x2*)vp;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          raw[2 * i] = (uint16_t)(x[i] & 0xffffu);
-          raw[2 * i + 1] = (uint16_t)(x[i] >> 16);
-        }
-      } else if constexpr (PER == 2) {
-        const uint32_t x = *(const uint32_t*)vp;
-        raw[0] = (uint16_t)(x & 0xffffu);
-        raw[1] = (uint16_t)(x >> 16);
-      } else {
-        raw[0] = *vp;
+      for (int i = 0; i < 4; ++i) {
+        raw[2 * i] = (uint16_t)(x[i] & 0xffffu);
+        raw[2 * i + 1] = (uint16_t)(x[i] >> 16);
       }
+    } else if constexpr (PER == 4) {
+      const u32x2 x = *(const u32x2*)vp;
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const float v = F16 ? (float)__builtin_bit_cast(_Float16, raw[i]) : bf16_bits_to_f32(raw[i]);
-        acc[i] = __builtin_fmaf(pj, v, acc[i]);
+      for (int i = 0; i < 2; ++i) {
+        raw[2 * i] = (uint16_t)(x[i] & 0xffffu);
+        raw[2 * i + 1] = (uint16_t)(x[i] >> 16);
+      }
+    } else if constexpr (PER == 2) {
+      const uint32_t x = *(const uint32_t*)vp;
+      raw[0] = (uint16_t)(x & 0xffffu);
+      raw[1] = (uint16_t)(x >> 16);
+    } else {
+      raw[0] = *vp;
+    }
+  };
+  for (uint32_t j0 = wave * GU; j0 < k; j0 += 4u * GU) {
+    float pj[GU];
+    uint16_t raw[GU][PER];
+#pragma unroll
+    for (int u = 0; u < GU; ++u) {
+      const uint32_t j = min(j0 + (uint32_t)u, k - 1u);          // past the end: the last key again, weight 0
+      pj[u] = j0 + (uint32_t)u < k ? sh.sel_s[j] * inv : 0.f;
+      const uint32_t tj = min(sh.sel_t[j], p.t_all - 1u);       // (kept positions are < t_all by construction)
+      const uint16_t* vp = (const uint16_t*)(vbase + (int64_t)kv_slot(p.ring_mask, tj) * vstride_b);
+      if (lane_on) load_row(vp, raw[u]);
+    }
+    if (lane_on) {
+#pragma unroll
+      for (int u = 0; u < GU; ++u) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const float v = F16 ? (float)__builtin_bit_cast(_Float16, raw[u][i]) : bf16_bits_to_f32(raw[u][i]);
+          acc[i] = __builtin_fmaf(pj[u], v, acc[i]);
+        }
       }
     }
   }
+  TK_PHASE(5)
   if (lane_on) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) red[wave][lane * PER + i] = acc[i];
@@ -545,32 +729,36 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
 }
 
 template <int D, bool F16>
-hipError_t launch_pair(const TopkParams& tp, hipStream_t s) {
-  const uint32_t n_units = tp.a.hkv * tp.n_splits * tp.n_mtiles;
-  const uint32_t grid = ((n_units + 7u) / 8u) * 8u;
-  hipLaunchKernelGGL((topk_scores_kernel<D, F16>), dim3(grid), dim3(256), 0, s, tp);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL((topk_select_kernel<D, F16>), dim3(tp.ntok, tp.a.hq), dim3(256), 0, s, tp);
+hipError_t launch_stage(const TopkParams& tp, int stage, hipStream_t s) {
+  if (stage == 0) {
+    const uint32_t n_units = tp.a.hkv * tp.n_splits * tp.n_mtiles;
+    const uint32_t grid = ((n_units + 7u) / 8u) * 8u;
+    hipLaunchKernelGGL((topk_scores_kernel<D, F16>), dim3(grid), dim3(256), 0, s, tp);
+  } else {
+    hipLaunchKernelGGL((topk_select_kernel<D, F16>), dim3(tp.ntok, tp.a.hq), dim3(256), 0, s, tp);
+  }
   return hipGetLastError();
 }
 
 template <bool F16>
-hipError_t launch_by_dim(const TopkParams& tp, uint32_t head_dim, hipStream_t s) {
+hipError_t launch_by_dim(const TopkParams& tp, int stage, uint32_t head_dim, hipStream_t s) {
   switch (head_dim) {
-    case 32: return launch_pair<32, F16>(tp, s);
-    case 64: return launch_pair<64, F16>(tp, s);
-    case 128: return launch_pair<128, F16>(tp, s);
-    case 256: return launch_pair<256, F16>(tp, s);
-    case 512: return launch_pair<512, F16>(tp, s);
+    case 32: return launch_stage<32, F16>(tp, stage, s);
+    case 64: return launch_stage<64, F16>(tp, stage, s);
+    case 128: return launch_stage<128, F16>(tp, stage, s);
+    case 256: return launch_stage<256, F16>(tp, stage, s);
+    case 512: return launch_stage<512, F16>(tp, stage, s);
     default: return hipErrorInvalidValue;
   }
 }
 
 }  // namespace
 
-hipError_t launch_attn_topk(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s) {
-  return kv_dtype == 1u ? launch_by_dim<true>(tp, head_dim, s) : launch_by_dim<false>(tp, head_dim, s);
+hipError_t launch_topk_scores(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s) {
+  return kv_dtype == 1u ? launch_by_dim<true>(tp, 0, head_dim, s) : launch_by_dim<false>(tp, 0, head_dim, s);
+}
+hipError_t launch_topk_select(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s) {
+  return kv_dtype == 1u ? launch_by_dim<true>(tp, 1, head_dim, s) : launch_by_dim<false>(tp, 1, head_dim, s);
 }
 
 }  // namespace dg

@@ -376,7 +376,10 @@ namespace {
 // Top-k sparse attention walks the canvas in row blocks so that the fp32 score plane of a block
 // ([Hq][rows][t_pad]) stays within the memory-side cache between the kernel that writes it and
 // the one that reads it.
-constexpr size_t kTopkPlaneBudget = 144ull << 20;
+#ifndef DG_TOPK_PLANE_MIB
+#define DG_TOPK_PLANE_MIB 144
+#endif
+constexpr size_t kTopkPlaneBudget = (size_t)DG_TOPK_PLANE_MIB << 20;
 
 struct TopkPlan {
   uint32_t t_pad = 0, block_tok = 0;
@@ -397,6 +400,7 @@ int make_topk_plan(const dg_attn_desc* d, const uint32_t* k_cfg, const Plan& pl,
   if (blk >= 16) blk &= ~(size_t)15;
   tk->block_tok = (uint32_t)std::min<size_t>(blk, d->canvas);
   tk->total = align_up((size_t)tk->block_tok * per_tok);
+  if (tk->total / sizeof(float) >= (1ull << 32)) return DG_ERR_SHAPE;   // score rows are addressed with 32-bit offsets
   return DG_OK;
 }
 }  // namespace
@@ -434,6 +438,9 @@ int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const voi
   rc = fill_params(d, pl, q, kv_base, out, nullptr, nullptr, s, &tp.a);   // no conversion passes: dtypes checked above
   if (rc != DG_OK) return rc;
   tp.a.dbg = g_tls_dbg;
+#ifdef DG_ATTN_PHASE_TIMING
+  tp.a.phase_cycles = g_phase_cycles;
+#endif
   tp.s_plane = (float*)workspace;
   tp.t_pad = tk.t_pad;
   tp.tile_first = pl.tile_first;
@@ -450,7 +457,19 @@ int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const voi
     const uint32_t base = d->n_kv_heads * tp.n_mtiles;
     uint32_t splits = std::max(1u, (256u + base - 1u) / base);
     tp.n_splits = std::max(1u, std::min(splits, ntiles / 8u));
-    if (dg::launch_attn_topk(tp, d->head_dim, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+    // (timing aid: one event pair per kernel, scores first)
+    const bool prof = g_prof.active && 2 * (size_t)g_prof.used + 3 < g_prof.ev.size();
+    if (prof) (void)hipEventRecord(g_prof.ev[2 * g_prof.used], s);
+    if (dg::launch_topk_scores(tp, d->head_dim, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+    if (prof) {
+      (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 1], s);
+      (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 2], s);
+    }
+    if (dg::launch_topk_select(tp, d->head_dim, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+    if (prof) {
+      (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 3], s);
+      g_prof.used += 2;
+    }
   }
   return DG_OK;
 }
@@ -529,23 +548,31 @@ int dg_prof_begin(uint32_t max_launches) {
   return DG_OK;
 }
 
-int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches) {
+int dg_prof_end_split(double* even_ms_total, double* odd_ms_total, uint32_t* n_pairs) {
   if (!g_prof.active) return DG_ERR_UNSUPPORTED;
-  double total = 0.0;
+  double total[2] = {0.0, 0.0};
   int rc = DG_OK;
   if (g_prof.used > 0 && hipEventSynchronize(g_prof.ev[2 * g_prof.used - 1]) != hipSuccess) rc = DG_ERR_LAUNCH;
   for (uint32_t i = 0; i < g_prof.used && rc == DG_OK; ++i) {
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]) != hipSuccess) rc = DG_ERR_LAUNCH;
-    total += ms;
+    total[i & 1u] += ms;
   }
   for (auto e : g_prof.ev)
     if (e) (void)hipEventDestroy(e);
-  if (main_kernel_ms_total) *main_kernel_ms_total = total;
-  if (n_launches) *n_launches = g_prof.used;
+  if (even_ms_total) *even_ms_total = total[0];
+  if (odd_ms_total) *odd_ms_total = total[1];
+  if (n_pairs) *n_pairs = g_prof.used;
   g_prof.ev.clear();
   g_prof.used = 0;
   g_prof.active = false;
+  return rc;
+}
+
+int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches) {
+  double even = 0.0, odd = 0.0;
+  const int rc = dg_prof_end_split(&even, &odd, n_launches);
+  if (main_kernel_ms_total) *main_kernel_ms_total = even + odd;
   return rc;
 }
 

@@ -242,6 +242,11 @@ int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void*
  * recorded event, returns the summed kernel time and releases the events. */
 int dg_prof_begin(uint32_t max_launches);
 int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches);
+/* dg_attn_topk_forward records two pairs per block of canvas rows instead: one around the score
+ * kernel, then one around the select kernel.  dg_prof_end_split ends the session like dg_prof_end
+ * and returns the time of the even-numbered pairs (0, 2, ...: the score kernels of a top-k
+ * session) and of the odd-numbered ones (the select kernels) separately. */
+int dg_prof_end_split(double* even_ms_total, double* odd_ms_total, uint32_t* n_pairs);
 
 /* Plain device-to-device copy of `bytes` (multiple of 16) with a kernel of this library: a
  * launch of known HBM traffic (bytes read + bytes written) that the FETCH_SIZE / WRITE_SIZE
