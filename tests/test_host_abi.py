@@ -108,6 +108,35 @@ def test_split_planning():
     assert capi.workspace_bytes(A.make_desc(2, 4, 2, 32, 2)) == 0
 
 
+def test_topk_planning_and_validation():
+    from diffgemma_amd import attention_topk as T
+    d = W.config("cfg3_global").desc()
+    # score plane of one block of canvas rows: 64 rows x 16 heads x 33024 keys (a multiple of 32) x fp32 <= 144 MiB
+    assert T.workspace_bytes(d, T.adaptive_k()) == 64 * 16 * 33024 * 4
+    small = A.make_desc(8, 4, 2, 64, 100)
+    assert T.workspace_bytes(small, T.fixed_k(64)) == 8 * 4 * 128 * 4            # whole canvas in one block, keys padded to 128
+    lib = capi.load()
+    n = C.c_size_t(0)
+    cfg = lambda *v: (C.c_uint32 * 4)(*v)
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(d), cfg(1025, 0, 0, 0), C.byref(n)) == capi.DG_ERR_SHAPE
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(d), cfg(1024, 0, 0, 0), C.byref(n)) == capi.DG_OK
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(d), cfg(256, 128, 64, 1025), C.byref(n)) == capi.DG_ERR_SHAPE
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(d), cfg(256, 128, 513, 512), C.byref(n)) == capi.DG_ERR_SHAPE
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(d), None, C.byref(n)) == capi.DG_ERR_NULL
+    scalar = A.make_desc(8, 4, 2, 64, 100, kernel=capi.DG_KERNEL_SCALAR)
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(scalar), cfg(8, 0, 0, 0), C.byref(n)) == capi.DG_ERR_UNSUPPORTED
+    f32 = A.make_desc(8, 4, 2, 64, 100, q_dtype=capi.DG_F32, kv_dtype=capi.DG_F32, out_dtype=capi.DG_F32)
+    assert lib.dg_attn_topk_workspace_bytes(C.byref(f32), cfg(8, 0, 0, 0), C.byref(n)) == capi.DG_ERR_UNSUPPORTED
+    # the reference-shaped size query agrees with the general one (bf16 Q, f16 cache, slot-major)
+    f = A.full_grp8_hd512_fixture()
+    lo, dims = A.layer_offsets(f), capi.AttnDims(canvas=f.canvas, n_q_heads=f.n_q_heads, causal=1, window=0)
+    assert lib.dg_attention_topk_state_bytes(C.byref(lo), C.byref(dims), f.kv_len, cfg(64, 0, 0, 0), C.byref(n)) == capi.DG_OK
+    t_pad = -(-(f.kv_len + f.canvas) // 32) * 32
+    assert n.value == f.canvas * f.n_q_heads * t_pad * 4
+    assert T.k_pad_for(1) == 64 and T.k_pad_for(65) == 128 and T.k_pad_for(5000) == 1024     # mod.rs:34-36
+    assert T.fixed_k(0) == (1, 0, 0, 0) and T.fixed_k(100) == (100, 0, 0, 0)
+
+
 def test_visible_pairs_and_flops():
     pairs, flops = capi.visible_pairs(W.config("cfg3_global").desc())
     assert pairs == 8429632 and flops == 4.0 * 512 * 16 * 8429632
