@@ -36,9 +36,18 @@ constexpr int kCandCap = 2048;     // LDS candidate list of the select kernel (s
     atomicAdd(&p.phase_cycles[i], now - tk_t);                             \
     tk_t = now;                                                            \
   }
+#define SC_PHASE(i)                                                        \
+  if (p.phase_cycles && threadIdx.x == 0) {                                \
+    const unsigned long long now = clock64();                              \
+    atomicAdd(&p.phase_cycles[8 + (i)], now - sc_t);                       \
+    sc_t = now;                                                            \
+  }
+#define SC_PHASE_DECL unsigned long long sc_t = clock64();
 #else
 #define TK_PHASE_DECL
 #define TK_PHASE(i)
+#define SC_PHASE(i)
+#define SC_PHASE_DECL
 #endif
 // radix digits of the 32-bit key, most significant first: 11 + 11 + 10 bits
 __device__ __forceinline__ uint32_t digit_shift(int level) { return level == 0 ? 21u : level == 1 ? 10u : 0u; }
@@ -153,26 +162,31 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
   // store instruction writes 32 consecutive keys of two rows: whole 128-byte lines.  (With the
   // operands the other way round every store scatters 32-byte pieces over 32 rows and the
   // kernel is bound by the write path.)  Where each of the 16 rows lives, and whether it exists:
-  uint32_t row_off[16];      // float offset of the row in the score plane, without the key
+  uint32_t row_off[16];      // byte offset of this lane's key column in the row, in the first key tile
   uint32_t row_mask = 0;
+  const bool full_tile = row0 + kBlockM <= rows_total;      // (the same in every lane)
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
     const uint32_t rr = row0 + wave * 32u + 8u * (e >> 2) + 4u * g2 + (e & 3);
     const bool ok = rr < rows_total;
     const uint32_t tl = ok ? rr / p.group : 0u;
     const uint32_t hh = kvh * p.group + (ok ? rr % p.group : 0u);
-    row_off[e] = (hh * tp.ntok + tl) * tp.t_pad;
+    row_off[e] = ((hh * tp.ntok + tl) * tp.t_pad + l32) * 4u;
     row_mask |= ok ? 1u << e : 0u;
   }
 
+  SC_PHASE_DECL
 #pragma unroll
   for (int i = 0; i < PF; ++i) issue_k(tb + i);
-  // lane l32 holds key t0 + l32 of sixteen rows
+  // lane l32 holds key t0 + l32 of sixteen rows; element e of a tile's scores goes to
+  // (uniform tile base) + (per-lane 32-bit offset)
+  auto store_elem = [&](auto e_c, const f32x16& sc, uint32_t tile) {
+    constexpr int e = decltype(e_c)::value;
+    char* const base = (char*)tp.s_plane + (size_t)tile * (kBlockN * sizeof(float));
+    if (full_tile || (row_mask & (1u << e))) *(float*)(base + row_off[e]) = sc[e] * tp.scale;
+  };
   auto store_tile = [&](const f32x16& sc, uint32_t tile) {
-    float* const dst = tp.s_plane + tile * kBlockN + l32;
-#pragma unroll
-    for (int e = 0; e < 16; ++e)
-      if (row_mask & (1u << e)) dst[row_off[e]] = sc[e] * tp.scale;
+    static_for<0, 16>([&](auto e_c) { store_elem(e_c, sc, tile); });
   };
   f32x16 s_prev;
 #pragma unroll
@@ -180,11 +194,14 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
   for (uint32_t j = tb; j < te; ++j) {
     // this wave's loads of K(j) have landed (the PF-1 tiles behind it may still be in flight);
     // after the barrier everybody's have, and everybody is done reading K(j-1), whose buffer
-    // takes K(j+PF).  The scores of tile j-1 are stored only now, a tile late: stores count in
-    // the same counter as the loads, and issued right before the wait they would have to drain
-    // first; issued here they are a tile old at the next wait.
+    // takes K(j+PF).  The scores of tile j-1 are stored only now, a tile late, between the
+    // first half of this tile's MFMAs: stores count in the same counter as the loads, and issued
+    // right before the wait they would have to drain first; issued here they are at least half
+    // a tile old at the next wait, and their address arithmetic hides behind the matrix pipe.
+    SC_PHASE(0)
     wait_loads_then_barrier<(PF - 1) * NLD>();
-    if (j > tb) store_tile(s_prev, j - 1u);
+    SC_PHASE(1)
+    const bool have_prev = j > tb;
     // (the loads of K(j+PF) are issued between the MFMAs below: back to back each of them holds
     // the wave's issue slot for about two MFMAs' worth of cycles)
     const TileLoad tl_next = k_desc(j + PF);
@@ -200,6 +217,8 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
     constexpr int LPC = (NLD + NCHUNK - 1) / NCHUNK;      // tile loads issued per chunk
     constexpr int LGAP = CH / LPC;                         // MFMAs between two of them
     static_assert(LPC * NCHUNK >= NLD && LPC <= CH, "tile loads must fit between the MFMAs");
+    constexpr int SHALF = NSTEP / 2 > 0 ? NSTEP / 2 : 1;   // MFMAs that carry stores of the previous tile
+    constexpr int SPM = (16 + SHALF - 1) / SHALF;          // stores behind each of them
     u32x4 fr[2][CH];
     auto read_chunk = [&](int c, u32x4 (&dst)[CH]) {
 #pragma unroll
@@ -225,12 +244,19 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
           issue_tile_part<D, false, c * LPC + i / LGAP>(tl_next, wave, lane);
           __builtin_amdgcn_sched_barrier(0);
         }
+        constexpr int m = c * CH + i;                 // MFMA index within the tile
+        if constexpr (m < SHALF) {
+          if (have_prev) static_for<m * SPM, (m + 1) * SPM < 16 ? (m + 1) * SPM : 16>([&](auto e_c) { store_elem(e_c, s_prev, j - 1u); });
+          __builtin_amdgcn_sched_barrier(0);
+        }
       });
       __builtin_amdgcn_sched_barrier(0);
     });
     s_prev = s;
+    SC_PHASE(2)
   }
   store_tile(s_prev, te - 1u);
+  SC_PHASE(3)
   wait_vmem_all();   // no direct-to-LDS load may outlive the workgroup's LDS
 }
 
