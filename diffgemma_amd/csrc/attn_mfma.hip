@@ -36,7 +36,7 @@
 // would rescale some row block on almost every tile.  Any reference below the true max is
 // exact as long as nothing overflows: P <= 2^tau, and the fp32 sums stay below
 // 2^tau * keys * |v|, far from 2^127 for tau = 80.  With f16 operands P itself has to stay
-// below 65504.
+// below 65504: tau = 15.
 #include "attn_params.h"
 #include "mfma_tile.h"
 
@@ -45,7 +45,7 @@ namespace {
 
 // log2 units by which a tile max may exceed the reference max before the reference is raised
 template <bool F16>
-constexpr float kTau = F16 ? 12.0f : 80.0f;
+constexpr float kTau = F16 ? 15.0f : 80.0f;
 
 // Optional per-phase cycle accounting (development builds only): every wave sums the cycles
 // it spends in each phase of the tile loop and stores the sums at the end.

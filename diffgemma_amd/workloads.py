@@ -39,6 +39,7 @@ class Workload:
     outlier_gain: float = 1.0
     seed: int = 0
     sees_masked: bool = False
+    kv_f16: bool = False             # cache stored as f16 under bf16 queries (the reference's own pairing)
 
     @property
     def t_all(self) -> int:
@@ -53,7 +54,8 @@ class Workload:
             t_lo = self.t_lo
         if self.sees_masked:
             flags |= capi.DG_ATTN_F_CAUSAL_SEES_MASKED
-        args = dict(causal_rows=self.causal_rows, window=self.window, q_dtype=dt, kv_dtype=dt,
+        args = dict(causal_rows=self.causal_rows, window=self.window, q_dtype=dt,
+                    kv_dtype=capi.DG_F16 if self.kv_f16 else dt,
                     out_dtype=dt, flags=flags, t_lo=t_lo, layout=self.layout, t_cap=self.t_all)
         args.update(kw)
         return make_desc(self.canvas, self.n_q_heads, self.n_kv_heads, self.head_dim, self.kv_len, **args)
@@ -72,6 +74,8 @@ def config(name: str) -> Workload:
         return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, seed=3)
     if name == "cfg3_global_b":       # committed rows additionally see canvas keys >= 128
         return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, sees_masked=True, seed=3)
+    if name == "cfg3_global_f16kv":   # config 3 with the reference's storage: bf16 activations, f16 cache
+        return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, seed=3, kv_f16=True)
     if name == "cfg4_long":
         return Workload(name, 256, 16, 2, 512, 131072, rms_norm=False, kv_std=0.5, outlier_frac=0.01,
                         outlier_gain=8.0, seed=4)
@@ -131,6 +135,11 @@ def generate(w: Workload) -> Tuple[np.ndarray, np.ndarray]:
             for h in range(w.n_kv_heads):
                 kv[plane, h] = rounding.bf16_bits_to_f32(rounding.f32_to_bf16_bits_rne(kv[plane, h])).reshape(
                     kv[plane, h].shape)
+        if w.kv_f16:   # bf16 values are f16 values unless they are tiny: flush those the way the store does
+            for plane in range(2):
+                for h in range(w.n_kv_heads):
+                    kv[plane, h] = rounding.f16_bits_to_f32(rounding.f32_to_f16_bits_rne(kv[plane, h])).reshape(
+                        kv[plane, h].shape)
     if w.layout == "reference":
         kv = np.ascontiguousarray(kv.transpose(2, 0, 1, 3))  # [T, 2, Hkv, hd]
     return q, kv
@@ -144,7 +153,8 @@ def device_arrays(w: Workload, q: np.ndarray, kv: np.ndarray):
         kd = torch.empty(kv.size, dtype=torch.int16, device="cuda")
         flat = kv.reshape(-1)
         step = 1 << 25
-        for o in range(0, flat.size, step):  # values are exactly representable: truncation is exact
-            kd[o:o + step] = torch.from_numpy(rounding.f32_to_bf16_bits_trunc(flat[o:o + step]).view(np.int16)).cuda()
+        to_bits = rounding.f32_to_f16_bits_rne if w.kv_f16 else rounding.f32_to_bf16_bits_trunc
+        for o in range(0, flat.size, step):  # values are exactly representable: the conversion is exact
+            kd[o:o + step] = torch.from_numpy(to_bits(flat[o:o + step]).view(np.int16)).cuda()
         return qd, kd
     return torch.from_numpy(q.reshape(-1)).cuda(), torch.from_numpy(kv.reshape(-1)).cuda()

@@ -124,7 +124,7 @@ def test_cfg2_sliding_window(gpu_ready, po, name):
     check_tolerances(*run_workload(po, W.config(name)))
 
 
-@pytest.mark.parametrize("name", ["cfg3_global", "cfg3_global_b"])
+@pytest.mark.parametrize("name", ["cfg3_global", "cfg3_global_b", "cfg3_global_f16kv"])
 def test_cfg3_global_full_size(gpu_ready, po, name):
     """Full 32k-prefix shape, every row, mixed committed/bidirectional mask."""
     check_tolerances(*run_workload(po, W.config(name)))
