@@ -58,7 +58,13 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
     po.attention_f32(d, q, kv, tok_list=toks, n_threads=threads)
     dt = time.perf_counter() - t0
     fl = float(sum(flops_per_tok[t] for t in toks))
+    # the same code on one thread, on the two probe rows
+    t0 = time.perf_counter()
+    po.attention_f32(d, q, kv, tok_list=probe, n_threads=1)
+    dt1 = max(time.perf_counter() - t0, 1e-4)
+    single = float(sum(flops_per_tok[int(t)] for t in probe)) / dt1 / 1e12
     return {"value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "single_thread_value": single,
             "sample": f"{len(toks)} of {w.canvas} canvas rows (evenly spaced) x all {w.n_q_heads} heads, "
                       f"{dt:.2f} s, fp32 online-softmax port of the reference CPU attention, OpenMP"}
 
