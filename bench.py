@@ -30,6 +30,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="cfg3_global")
+    ap.add_argument("--global-topk", action="store_true",
+                    help="cfg5_schedule: run the global layers as top-k sparse attention (the reference's default for them)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline sample time")
@@ -152,9 +154,11 @@ def bench_schedule(args):
     layers (Hkv 2, hd 512) at indices 5, 11, 17, 23, 29; the canvas projections are regenerated on the
     device before every iteration, the prefix rows stay."""
     import torch
-    from diffgemma_amd import attention as A, capi, qk_rope_kv as QR, rounding as R, step_kv
+    from diffgemma_amd import attention as A, attention_topk as T, capi, qk_rope_kv as QR, rounding as R, step_kv
     from oracle import pyoracle as po
     canvas, nq, kv_len, ring = 256, 16, 32768, 2048
+    k_cfg = T.adaptive_k()
+    topk_ws = None
     lib = capi.load()
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1234)
@@ -186,6 +190,8 @@ def bench_schedule(args):
                "kw": A.to_device_bits(R.f32_to_bf16_bits_rne(f.k_norm_w)),
                "out": torch.zeros(canvas * nq * hd, dtype=torch.int16, device="cuda"),
                "ws": A.alloc_workspace(ad)}
+        if full and args.global_topk and topk_ws is None:
+            topk_ws = T.alloc_workspace(ad, k_cfg)      # one score plane, shared by the global layers
         layers.append(lay)
         flops_iter += capi.visible_pairs(ad)[1]
 
@@ -202,7 +208,10 @@ def bench_schedule(args):
             capi.check(lib.dg_qk_rope_kv(C.byref(lay["rd"]), lay["q"].data_ptr(), lay["k"].data_ptr(),
                                          lay["v"].data_ptr(), lay["cache"].data_ptr(), lay["qw"].data_ptr(),
                                          lay["kw"].data_ptr(), None, st))
-            A.forward(lay["ad"], lay["q"], lay["cache"], lay["out"], None, lay["ws"])
+            if lay["full"] and args.global_topk:
+                T.forward(lay["ad"], k_cfg, lay["q"], lay["cache"], lay["out"], topk_ws)
+            else:
+                A.forward(lay["ad"], lay["q"], lay["cache"], lay["out"], None, lay["ws"])
 
     regenerate(0)
     side = torch.cuda.Stream()
@@ -231,7 +240,10 @@ def bench_schedule(args):
         od = po.make_desc(canvas, nq, nkv, hd, kv_len, window=0 if lay["full"] else 1024,
                           kv_ring_mask=0 if lay["full"] else ring - 1, layout="head_major", t_cap=slots)
         toks = np.array([0, 100, 255], dtype=np.uint32)
-        ref, _ = po.attention_f32(od, qh, kvh, tok_list=toks)
+        if lay["full"] and args.global_topk:
+            ref = po.attention_topk_f32(od, k_cfg, qh, kvh, tok_list=toks)
+        else:
+            ref, _ = po.attention_f32(od, qh, kvh, tok_list=toks)
         got = R.bf16_bits_to_f32(lay["out"].cpu().numpy().view(np.uint16)).reshape(canvas, nq, hd)
         d = np.abs(got[toks] - ref[toks])
         check["layers"][str(idx)] = {"max_abs": float(d.max()), "mean_abs": float(d.mean())}
@@ -259,7 +271,9 @@ def bench_schedule(args):
            "dtype": "bf16", "data": "synthetic",
            "config": {"workload": "cfg5_schedule", "layers": step_kv.N_LAYERS, "global_layers": list(step_kv.FULL_LAYERS),
                       "canvas": canvas, "kv_prefix": kv_len, "sliding": "Hq16/Hkv8 hd256 window 1024 ring 2048",
-                      "global": "Hq16/Hkv2 hd512", "kv_layout": "bf16 head-major planes", "launch": "HIP graph, 120 kernels"},
+                      "global": "Hq16/Hkv2 hd512" + (", top-k sparse attention, k = t/128 (FLOP/s counted as if dense)"
+                                                    if args.global_topk else ", dense"),
+                      "kv_layout": "bf16 head-major planes", "launch": "HIP graph"},
            "flops_per_step": flops_iter, "canvas_tokens_per_s": canvas / (ms * 1e-3),
            "iteration_ms": {"min": per_iter[0], "median": per_iter[len(per_iter) // 2], "max": per_iter[-1]},
            "roofline": None, "cpu_baseline": None, "check": check}
