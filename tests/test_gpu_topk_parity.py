@@ -163,6 +163,53 @@ def test_global_layer_at_32k_prefix_rows(gpu_ready, po):
     assert max_abs_diff(got[toks], ref[toks]) <= 2e-2 and mean_abs_diff(got[toks], ref[toks]) <= 2e-3
 
 
+# ------------------------------------------------------------------ edge cases
+EDGE = [
+    # canvas, hq, hkv, hd, kv_len, causal_rows, window, k_cfg
+    (1, 4, 2, 64, 0, 1, 0, (8, 0, 0, 0)),              # one row, one key
+    (1, 16, 2, 512, 77, 0, 0, T.adaptive_k()),          # single denoise row, fewer keys than k_min
+    (5, 2, 1, 32, 3, 0, 0, (1, 0, 0, 0)),               # less than one key tile in total
+    (37, 12, 4, 64, 333, 20, 100, (17, 0, 0, 0)),       # ragged everything: group 3, mixed rows, window
+    (256, 16, 8, 256, 0, 256, 0, T.adaptive_k()),       # prefill from an empty cache, per-row k
+    (64, 16, 2, 512, 40000, 64, 0, (256, 128, 64, 512)),  # two blocks of canvas rows (score plane budget)
+    (8, 8, 8, 128, 5000, 0, 0, (600, 0, 0, 0)),         # no GQA sharing
+]
+
+
+@pytest.mark.parametrize("case", EDGE)
+def test_edge_cases(gpu_ready, po, case):
+    canvas, hq, hkv, hd, kvl, cr, win, k_cfg = case
+    toks = None if canvas <= 64 else np.unique(np.linspace(0, canvas - 1, 16).round().astype(np.uint32))
+    got, ref = run_topk(po, canvas, hq, hkv, hd, kvl, k_cfg, causal_rows=cr, window=win, seed=hash(case[:7]) & 0xFFFF,
+                        toks=toks)
+    assert np.isfinite(got).all()
+    assert max_abs_diff(got, ref) <= 2e-2 and mean_abs_diff(got, ref) <= 2e-3
+
+
+def test_ring_cache(gpu_ready, po):
+    """Top-k over a wrapped ring (a sliding layer's storage): kept positions map to slots for the gather."""
+    import torch
+    canvas, hq, hkv, hd, kvl, window, ring, k = 32, 4, 2, 128, 3000, 1000, 2048, 40
+    rng = np.random.default_rng(77)
+    t_all = kvl + canvas
+    q = rng.standard_normal((canvas, hq, hd)).astype(np.float32)
+    lin = rng.standard_normal((t_all, 2, hkv, hd)).astype(np.float32)
+    qb, lb = R.f32_to_bf16_bits_rne(q), R.f32_to_bf16_bits_rne(lin).reshape(lin.shape)
+    ringbits = np.full((ring, 2, hkv, hd), 0x7FC0, dtype=np.uint16)          # NaN in every dead slot
+    for pos in range(kvl - (window - 1), t_all):
+        ringbits[pos & (ring - 1)] = lb[pos]
+    d = A.make_desc(canvas, hq, hkv, hd, kvl, window=window, kv_ring_mask=ring - 1, out_dtype=capi.DG_F32)
+    out = torch.zeros(canvas * hq * hd, dtype=torch.float32, device="cuda")
+    cfg = (k, 0, 0, 0)
+    T.forward(d, cfg, A.to_device_bits(qb.reshape(-1)), A.to_device_bits(ringbits.reshape(-1)), out, T.alloc_workspace(d, cfg))
+    torch.cuda.synchronize()
+    od = po.make_desc(canvas, hq, hkv, hd, kvl, window=window)
+    ref = po.attention_topk_f32(od, cfg, R.bf16_bits_to_f32(qb).reshape(q.shape), R.bf16_bits_to_f32(lb).reshape(lin.shape))
+    got = out.cpu().numpy().reshape(ref.shape)
+    assert np.isfinite(got).all()
+    assert max_abs_diff(got, ref) <= 2e-2 and mean_abs_diff(got, ref) <= 2e-3
+
+
 # ------------------------------------------------------------------ properties
 def test_k_at_least_the_visible_keys_is_dense_attention(gpu_ready):
     import torch
