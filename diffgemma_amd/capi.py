@@ -29,6 +29,8 @@ EXPORTS = (
     "dg_calib_copy", "dg_calib_mfma", "dg_qk_rope_kv", "dg_qk_rope_kv_dispatch",
     "dg_attn_topk_workspace_bytes", "dg_attn_topk_forward", "dg_attention_topk_state_bytes",
     "dg_attention_topk_dispatch", "dg_prof_end_split",
+    "dg_kv_layer_reference_layout", "dg_kv_layer_head_major_layout", "dg_kv_snapshot_bytes", "dg_kv_snapshot_gather",
+    "dg_kv_snapshot_scatter", "dg_kv_live_bytes", "dg_kv_live_gather", "dg_fnv1a64",
 )
 
 
@@ -51,6 +53,16 @@ class RopeDesc(C.Structure):
         ("kv_len", C.c_uint32), ("kv_write_end", C.c_uint32), ("kv_ring_mask", C.c_uint32), ("is_full", C.c_uint32),
         ("v_from_k", C.c_uint32), ("kv_dtype", C.c_uint32), ("flags", C.c_uint32), ("reserved", C.c_uint32),
         ("kv_region_bytes", C.c_uint64),
+        ("k_tok_stride", C.c_int64), ("k_head_stride", C.c_int64),
+        ("v_base_off", C.c_int64), ("v_tok_stride", C.c_int64), ("v_head_stride", C.c_int64),
+    ]
+
+
+class KvLayer(C.Structure):
+    """dg_kv_layer: one layer's region of the KV cache, for the snapshot calls."""
+    _fields_ = [
+        ("kv_region_bytes", C.c_uint64), ("n_kv_heads", C.c_uint32), ("head_dim", C.c_uint32),
+        ("slots", C.c_uint32), ("kv_ring_mask", C.c_uint32), ("kv_dtype", C.c_uint32), ("reserved", C.c_uint32),
         ("k_tok_stride", C.c_int64), ("k_head_stride", C.c_int64),
         ("v_base_off", C.c_int64), ("v_tok_stride", C.c_int64), ("v_head_stride", C.c_int64),
     ]
@@ -161,6 +173,22 @@ def load():
     lib.dg_prof_begin.restype = C.c_int
     lib.dg_prof_end.argtypes = [P(C.c_double), P(C.c_uint32)]
     lib.dg_prof_end.restype = C.c_int
+    lib.dg_kv_layer_reference_layout.argtypes = [P(KvLayer)]
+    lib.dg_kv_layer_reference_layout.restype = None
+    lib.dg_kv_layer_head_major_layout.argtypes = [P(KvLayer)]
+    lib.dg_kv_layer_head_major_layout.restype = None
+    lib.dg_kv_snapshot_bytes.argtypes = [P(KvLayer), C.c_uint32, C.c_uint64, P(C.c_uint64), P(C.c_uint64)]
+    lib.dg_kv_snapshot_bytes.restype = C.c_int
+    lib.dg_kv_snapshot_gather.argtypes = [VP, P(KvLayer), C.c_uint32, C.c_uint64, VP, C.c_size_t, VP]
+    lib.dg_kv_snapshot_gather.restype = C.c_int
+    lib.dg_kv_snapshot_scatter.argtypes = [VP, P(KvLayer), C.c_uint32, C.c_uint64, VP, C.c_size_t, VP]
+    lib.dg_kv_snapshot_scatter.restype = C.c_int
+    lib.dg_kv_live_bytes.argtypes = [P(KvLayer), C.c_uint32, C.c_uint64, C.c_uint32, P(C.c_uint64)]
+    lib.dg_kv_live_bytes.restype = C.c_int
+    lib.dg_kv_live_gather.argtypes = [VP, P(KvLayer), C.c_uint32, C.c_uint64, C.c_uint32, VP, C.c_size_t, VP]
+    lib.dg_kv_live_gather.restype = C.c_int
+    lib.dg_fnv1a64.argtypes = [VP, C.c_size_t, C.c_uint64]
+    lib.dg_fnv1a64.restype = C.c_uint64
     lib.dg_prof_end_split.argtypes = [P(C.c_double), P(C.c_double), P(C.c_uint32)]
     lib.dg_prof_end_split.restype = C.c_int
     _lib = lib

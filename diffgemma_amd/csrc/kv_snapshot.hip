@@ -1,0 +1,237 @@
+// KV-cache snapshots for gfx950 (MI355X): the live part of every layer's region copied between
+// the cache, in whatever layout the kernels read it, and a compact blob in the reference's
+// snapshot format, so that conversation swap, rewinds and fingerprints see the same bytes
+// whichever layout the cache uses.
+//
+// Reference: gather_kv_prefix / scatter_kv_prefix (src/metal/step_kv/mod.rs:108-151: per layer
+// the first min(kv_len, slots) physical slots, each [K: Hkv x hd | V: Hkv x hd], layers
+// concatenated) and StepRuntime::live_kv_fnv (src/metal/step_kernel/runtime.rs:118-148: FNV-1a
+// over the readable state: linear layers their [0, kv_len) prefix, ring layers the last
+// min(kv_len, window) positions in position order).  There both are host loops over unified
+// memory; here the bytes are moved on the device by one kernel (16 bytes per lane, rows of
+// head_dim elements, any strided layout on the cache side) and the hash, a serial recurrence by
+// definition, runs on the host over the gathered stream.
+#include "../../include/dg_attn.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+
+namespace {
+
+constexpr int kMaxLayersPerLaunch = 32;
+
+struct MoveLayer {
+  uint64_t region_b;    // byte offset of the layer's region in the cache buffer
+  uint64_t blob_off;    // byte offset of the layer's rows in the blob
+  int64_t k_tok_b, k_head_b, v_base_b, v_tok_b, v_head_b;   // byte strides / offset inside the region
+  uint32_t hkv, row_bytes;   // one row = head_dim elements of one (position, K|V, head)
+  uint32_t first, count;     // positions [first, first + count)
+  uint32_t ring_mask;        // 0: slot = position
+  uint32_t pad;
+};
+
+struct MoveParams {
+  MoveLayer layer[kMaxLayersPerLaunch];
+  char* cache;
+  char* blob;
+  uint32_t to_blob;     // 1: cache -> blob, 0: blob -> cache
+};
+
+// blob rows of a layer, in order: position, then K | V, then head; a lane moves 16 bytes
+__global__ void __launch_bounds__(256) kv_move_kernel(const MoveParams p) {
+  const MoveLayer& L = p.layer[blockIdx.y];
+  const uint32_t cpr = L.row_bytes >> 4;                       // 16-byte chunks per row
+  const uint64_t n_chunks = (uint64_t)L.count * 2u * L.hkv * cpr;
+  for (uint64_t c = (uint64_t)blockIdx.x * 256u + threadIdx.x; c < n_chunks; c += (uint64_t)gridDim.x * 256u) {
+    const uint64_t row = c / cpr;
+    const uint32_t w = (uint32_t)(c % cpr);
+    const uint32_t head = (uint32_t)(row % L.hkv);
+    const uint32_t plane = (uint32_t)((row / L.hkv) & 1u);
+    const uint32_t pos = L.first + (uint32_t)(row / (2u * L.hkv));
+    const uint32_t slot = L.ring_mask ? (pos & L.ring_mask) : pos;
+    char* in_cache = p.cache + L.region_b +
+                     (plane ? L.v_base_b + (int64_t)slot * L.v_tok_b + (int64_t)head * L.v_head_b
+                            : (int64_t)slot * L.k_tok_b + (int64_t)head * L.k_head_b) +
+                     (uint64_t)w * 16u;
+    char* in_blob = p.blob + L.blob_off + row * L.row_bytes + (uint64_t)w * 16u;
+    if (p.to_blob) *(uint4*)in_blob = *(const uint4*)in_cache;
+    else *(uint4*)in_cache = *(const uint4*)in_blob;
+  }
+}
+
+uint32_t elem_bytes(uint32_t dtype) { return dtype == DG_F32 ? 4u : 2u; }
+
+int check_layer(const dg_kv_layer& l) {
+  if (l.n_kv_heads == 0 || l.head_dim == 0 || l.slots == 0) return DG_ERR_SHAPE;
+  if (l.kv_dtype > DG_F32) return DG_ERR_DTYPE;
+  const uint64_t row_b = (uint64_t)l.head_dim * elem_bytes(l.kv_dtype);
+  if (row_b % 16 != 0 || row_b > 0xffffffffull) return DG_ERR_SHAPE;
+  if (l.kv_ring_mask != 0 && ((((uint64_t)l.kv_ring_mask + 1) & l.kv_ring_mask) != 0 || l.kv_ring_mask >= l.slots))
+    return DG_ERR_LAYOUT;
+  const int64_t s[5] = {l.k_tok_stride, l.k_head_stride, l.v_base_off, l.v_tok_stride, l.v_head_stride};
+  for (int64_t x : s)
+    if (x < 0 || (x * (int64_t)elem_bytes(l.kv_dtype)) % 16 != 0) return DG_ERR_LAYOUT;
+  if (l.kv_region_bytes % 16 != 0) return DG_ERR_LAYOUT;
+  if (l.k_tok_stride < (int64_t)l.head_dim || l.v_tok_stride < (int64_t)l.head_dim) return DG_ERR_LAYOUT;
+  return DG_OK;
+}
+
+// positions a layer contributes: the snapshot takes physical slots [0, min(kv_len, slots)) as they
+// lie (no ring map); the live stream takes linear layers' [0, kv_len) and ring layers' last
+// min(kv_len, window) positions through the ring map
+struct Span {
+  uint32_t first, count, ring_mask;
+};
+
+int span_of(const dg_kv_layer& l, uint64_t kv_len, bool live, uint32_t window, Span* s) {
+  if (!live) {
+    s->first = 0;
+    s->count = (uint32_t)std::min<uint64_t>(kv_len, l.slots);
+    s->ring_mask = 0;
+    return DG_OK;
+  }
+  if (kv_len > 0xffffffffull) return DG_ERR_SHAPE;
+  if (l.kv_ring_mask == 0) {
+    if (kv_len > l.slots) return DG_ERR_SHAPE;
+    s->first = 0;
+    s->count = (uint32_t)kv_len;
+    s->ring_mask = 0;
+  } else {
+    const uint32_t n = (uint32_t)std::min<uint64_t>(kv_len, window);
+    if (n > l.slots) return DG_ERR_LAYOUT;   // the ring cannot hold a window's worth of positions
+    s->first = (uint32_t)kv_len - n;
+    s->count = n;
+    s->ring_mask = l.kv_ring_mask;
+  }
+  return DG_OK;
+}
+
+uint64_t layer_bytes(const dg_kv_layer& l, uint32_t count) {
+  return (uint64_t)count * 2u * l.n_kv_heads * l.head_dim * elem_bytes(l.kv_dtype);
+}
+
+int plan_bytes(const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len, bool live, uint32_t window,
+               uint64_t* total, uint64_t* offsets) {
+  if (!layers || !total) return DG_ERR_NULL;
+  uint64_t off = 0;
+  for (uint32_t i = 0; i < n_layers; ++i) {
+    int rc = check_layer(layers[i]);
+    if (rc != DG_OK) return rc;
+    Span s;
+    rc = span_of(layers[i], kv_len, live, window, &s);
+    if (rc != DG_OK) return rc;
+    if (offsets) offsets[i] = off;
+    off += layer_bytes(layers[i], s.count);
+  }
+  *total = off;
+  return DG_OK;
+}
+
+int move(void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len, bool live, uint32_t window,
+         void* blob, size_t blob_bytes, bool to_blob, void* stream) {
+  if (!kv_base) return DG_ERR_NULL;
+  uint64_t total = 0;
+  int rc = plan_bytes(layers, n_layers, kv_len, live, window, &total, nullptr);
+  if (rc != DG_OK) return rc;
+  if (total == 0) return DG_OK;            // nothing live yet: an empty blob may be a null pointer
+  if (!blob) return DG_ERR_NULL;
+  if (blob_bytes < total) return DG_ERR_WORKSPACE;
+  if (((uintptr_t)kv_base % 16) != 0 || ((uintptr_t)blob % 16) != 0) return DG_ERR_LAYOUT;
+  uint64_t off = 0;
+  for (uint32_t l0 = 0; l0 < n_layers; l0 += kMaxLayersPerLaunch) {
+    MoveParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.cache = (char*)kv_base;
+    p.blob = (char*)blob;
+    p.to_blob = to_blob ? 1u : 0u;
+    const uint32_t n = std::min<uint32_t>(kMaxLayersPerLaunch, n_layers - l0);
+    uint64_t max_chunks = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+      const dg_kv_layer& l = layers[l0 + i];
+      const int64_t eb = elem_bytes(l.kv_dtype);
+      Span s;
+      (void)span_of(l, kv_len, live, window, &s);
+      MoveLayer& m = p.layer[i];
+      m.region_b = l.kv_region_bytes;
+      m.blob_off = off;
+      m.k_tok_b = l.k_tok_stride * eb;
+      m.k_head_b = l.k_head_stride * eb;
+      m.v_base_b = l.v_base_off * eb;
+      m.v_tok_b = l.v_tok_stride * eb;
+      m.v_head_b = l.v_head_stride * eb;
+      m.hkv = l.n_kv_heads;
+      m.row_bytes = (uint32_t)(l.head_dim * eb);
+      m.first = s.first;
+      m.count = s.count;
+      m.ring_mask = s.ring_mask;
+      off += layer_bytes(l, s.count);
+      max_chunks = std::max<uint64_t>(max_chunks, layer_bytes(l, s.count) / 16u);
+    }
+    if (max_chunks == 0) continue;
+    const uint32_t bx = (uint32_t)std::min<uint64_t>((max_chunks + 255u) / 256u, 2048u);
+    hipLaunchKernelGGL(kv_move_kernel, dim3(bx, n), dim3(256), 0, (hipStream_t)stream, p);
+    if (hipGetLastError() != hipSuccess) return DG_ERR_LAUNCH;
+  }
+  return DG_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+void dg_kv_layer_reference_layout(dg_kv_layer* l) {
+  const int64_t row = (int64_t)l->n_kv_heads * l->head_dim;
+  l->k_tok_stride = 2 * row;
+  l->k_head_stride = l->head_dim;
+  l->v_base_off = row;
+  l->v_tok_stride = 2 * row;
+  l->v_head_stride = l->head_dim;
+}
+
+void dg_kv_layer_head_major_layout(dg_kv_layer* l) {
+  l->k_tok_stride = l->head_dim;
+  l->k_head_stride = (int64_t)l->slots * l->head_dim;
+  l->v_base_off = (int64_t)l->n_kv_heads * l->slots * l->head_dim;
+  l->v_tok_stride = l->head_dim;
+  l->v_head_stride = (int64_t)l->slots * l->head_dim;
+}
+
+int dg_kv_snapshot_bytes(const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len, uint64_t* total_bytes,
+                         uint64_t* layer_offsets) {
+  return plan_bytes(layers, n_layers, kv_len, false, 0, total_bytes, layer_offsets);
+}
+
+int dg_kv_snapshot_gather(const void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len,
+                          void* blob, size_t blob_bytes, void* stream) {
+  return move((void*)kv_base, layers, n_layers, kv_len, false, 0, blob, blob_bytes, true, stream);
+}
+
+int dg_kv_snapshot_scatter(void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len,
+                           const void* blob, size_t blob_bytes, void* stream) {
+  return move(kv_base, layers, n_layers, kv_len, false, 0, (void*)blob, blob_bytes, false, stream);
+}
+
+int dg_kv_live_bytes(const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len, uint32_t window,
+                     uint64_t* total_bytes) {
+  return plan_bytes(layers, n_layers, kv_len, true, window, total_bytes, nullptr);
+}
+
+int dg_kv_live_gather(const void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len,
+                      uint32_t window, void* stream_bytes, size_t capacity, void* stream) {
+  return move((void*)kv_base, layers, n_layers, kv_len, true, window, stream_bytes, capacity, true, stream);
+}
+
+uint64_t dg_fnv1a64(const void* bytes, size_t n, uint64_t seed_hash) {
+  const unsigned char* b = (const unsigned char*)bytes;
+  uint64_t h = seed_hash;
+  for (size_t i = 0; i < n; ++i) {
+    h ^= b[i];
+    h *= 0x00000100000001b3ull;
+  }
+  return h;
+}
+
+}  // extern "C"

@@ -6,8 +6,9 @@ global layers linear (+8 pad slots), sliding layers a power-of-two ring.
 """
 from __future__ import annotations
 
+import ctypes as C
 from dataclasses import dataclass
-from typing import List
+from typing import List, Sequence
 
 from . import capi
 
@@ -69,3 +70,61 @@ def build_layout(max_seq: int, kv_dtype: int = capi.DG_F16, ring_slots: int = KV
 
 def kv_cache_total_bytes(layers: List[LayerKv], kv_dtype: int = capi.DG_F16) -> int:
     return sum(kv_region_bytes(l.n_kv_heads, l.head_dim, l.slots, kv_dtype) for l in layers)
+
+
+# ---------------------------------------------------------------------------------------
+# snapshots and the live-KV fingerprint (src/metal/step_kv/mod.rs:108-151,
+# src/metal/step_kernel/runtime.rs:118-148), on a device buffer in either layout
+# ---------------------------------------------------------------------------------------
+
+def kv_layers(layers: Sequence[LayerKv], kv_dtype: int = capi.DG_F16, layout: str = "reference"):
+    """The dg_kv_layer array the snapshot calls take."""
+    lib = capi.load()
+    arr = (capi.KvLayer * len(layers))()
+    for a, l in zip(arr, layers):
+        a.kv_region_bytes, a.n_kv_heads, a.head_dim = l.kv_region, l.n_kv_heads, l.head_dim
+        a.slots, a.kv_ring_mask, a.kv_dtype = l.slots, l.kv_ring_mask, kv_dtype
+        if layout == "reference":
+            lib.dg_kv_layer_reference_layout(C.byref(a))
+        elif layout == "head_major":
+            lib.dg_kv_layer_head_major_layout(C.byref(a))
+        else:
+            raise ValueError(layout)
+    return arr
+
+
+def snapshot_bytes(arr, kv_len: int) -> int:
+    n = C.c_uint64(0)
+    capi.check(capi.load().dg_kv_snapshot_bytes(arr, len(arr), kv_len, C.byref(n), None))
+    return n.value
+
+
+def _stream() -> int:
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def gather_kv_prefix(buf, arr, kv_len: int):
+    """Compact blob (device uint8 tensor) of the live [0, kv_len) KV of every layer."""
+    import torch
+    blob = torch.empty(max(snapshot_bytes(arr, kv_len), 16), dtype=torch.uint8, device="cuda")
+    capi.check(capi.load().dg_kv_snapshot_gather(buf.data_ptr(), arr, len(arr), kv_len, blob.data_ptr(), blob.numel(),
+                                                 _stream()))
+    return blob[:snapshot_bytes(arr, kv_len)]
+
+
+def scatter_kv_prefix(buf, arr, kv_len: int, blob) -> None:
+    capi.check(capi.load().dg_kv_snapshot_scatter(buf.data_ptr(), arr, len(arr), kv_len, blob.data_ptr(), blob.numel(),
+                                                  _stream()))
+
+
+def live_kv_fnv(buf, arr, kv_len: int, seed_hash: int, window: int = SLIDING_WINDOW) -> int:
+    """FNV-1a over the readable KV state: the live stream is gathered on the device, copied to the host, hashed there."""
+    import torch
+    lib = capi.load()
+    n = C.c_uint64(0)
+    capi.check(lib.dg_kv_live_bytes(arr, len(arr), kv_len, window, C.byref(n)))
+    dev = torch.empty(max(n.value, 16), dtype=torch.uint8, device="cuda")
+    capi.check(lib.dg_kv_live_gather(buf.data_ptr(), arr, len(arr), kv_len, window, dev.data_ptr(), dev.numel(), _stream()))
+    host = dev[:n.value].cpu().numpy()
+    return int(lib.dg_fnv1a64(host.ctypes.data_as(C.c_void_p) if host.size else None, host.size, seed_hash))

@@ -267,6 +267,46 @@ uint64_t dg_kv_region_bytes(uint32_t n_kv_heads, uint32_t head_dim, uint64_t slo
 uint64_t dg_kv_slot(uint32_t kv_ring_mask, uint64_t pos);
 uint64_t dg_layer_kv_slots(int is_full, uint64_t max_seq, uint64_t ring_slots_cap);
 
+/* ---- KV-cache snapshots: the live part of every layer's region <-> a compact blob ----
+ *
+ * Replaces gather_kv_prefix / scatter_kv_prefix (src/metal/step_kv/mod.rs:108-151) and the byte
+ * walk of StepRuntime::live_kv_fnv (src/metal/step_kernel/runtime.rs:118-148), which in the
+ * reference are host loops over unified memory.  The blob keeps the reference's format whatever
+ * layout the cache uses: layers concatenated; per layer, position after position, a row of
+ * [K: Hkv x head_dim | V: Hkv x head_dim] elements.  A snapshot takes the first
+ * min(kv_len, slots) physical slots of a layer as they lie (ring layers too); the live stream is
+ * what the fingerprint hashes: linear layers their positions [0, kv_len), ring layers their last
+ * min(kv_len, window) positions in position order.  All pointers are device pointers; the calls
+ * enqueue one kernel per 32 layers on `stream` and return. */
+typedef struct dg_kv_layer {
+  uint64_t kv_region_bytes;  /* byte offset of the layer's region inside kv_base (LayerOffsets.kv_region) */
+  uint32_t n_kv_heads, head_dim;
+  uint32_t slots;            /* capacity of the region in positions (layer_kv_slots) */
+  uint32_t kv_ring_mask;     /* 0 = linear */
+  uint32_t kv_dtype;         /* DG_F16 / DG_BF16 / DG_F32 */
+  uint32_t reserved;
+  /* element strides/offsets inside the region, as in dg_attn_desc */
+  int64_t  k_tok_stride, k_head_stride;
+  int64_t  v_base_off, v_tok_stride, v_head_stride;
+} dg_kv_layer;
+void dg_kv_layer_reference_layout(dg_kv_layer* l);   /* [slot][K heads | V heads] */
+void dg_kv_layer_head_major_layout(dg_kv_layer* l);  /* K plane [Hkv][slots][hd], then V plane */
+
+/* layer_offsets (n_layers entries, may be NULL) receives each layer's byte offset in the blob */
+int dg_kv_snapshot_bytes(const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len, uint64_t* total_bytes,
+                         uint64_t* layer_offsets);
+int dg_kv_snapshot_gather(const void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len,
+                          void* blob, size_t blob_bytes, void* stream);
+int dg_kv_snapshot_scatter(void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len,
+                           const void* blob, size_t blob_bytes, void* stream);
+int dg_kv_live_bytes(const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len, uint32_t window,
+                     uint64_t* total_bytes);
+int dg_kv_live_gather(const void* kv_base, const dg_kv_layer* layers, uint32_t n_layers, uint64_t kv_len,
+                      uint32_t window, void* stream_bytes, size_t capacity, void* stream);
+/* FNV-1a over host bytes, continuing seed_hash (runtime.rs:127-133); the hash is a serial
+ * recurrence, so the fingerprint is dg_kv_live_gather + a copy to the host + this. */
+uint64_t dg_fnv1a64(const void* bytes, size_t n, uint64_t seed_hash);
+
 #ifdef __cplusplus
 }
 #endif

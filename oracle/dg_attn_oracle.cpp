@@ -245,6 +245,16 @@ void dgo_attention_topk_f32(const dgo_desc* dp, const uint32_t k_cfg[4], const f
   }
 }
 
+// FNV-1a, continuing seed_hash: src/metal/step_kernel/runtime.rs:127-133.
+uint64_t dgo_fnv1a64(const uint8_t* bytes, size_t n, uint64_t seed_hash) {
+  uint64_t h = seed_hash;
+  for (size_t i = 0; i < n; ++i) {
+    h ^= (uint64_t)bytes[i];
+    h *= 0x00000100000001b3ull;
+  }
+  return h;
+}
+
 void dgo_attention_f64(const dgo_desc* dp, const float* q, const float* kv, double* out, double* lse,
                        const uint32_t* tok_list, uint32_t n_tok, int n_threads) {
   const dgo_desc d = *dp;

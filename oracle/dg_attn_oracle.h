@@ -18,6 +18,10 @@
  *                            lower index, softmax over the kept keys, V summed in selection order);
  *   dgo_topk_row_k           src/shaders/attn/attention_topk/attention_topk.metal:160-182 (fixed or
  *                            context-adaptive k per row), src/flags/accessors.rs:210-221 (k_cfg)
+ *   dgo_fnv1a64              src/metal/step_kernel/runtime.rs:127-133 (FNV-1a, 64 bit); the snapshot gather /
+ *                            scatter and the live-KV byte walk (src/metal/step_kv/mod.rs:108-151,
+ *                            runtime.rs:118-148) are restated in numpy in pyoracle.py (kv_gather_prefix,
+ *                            kv_scatter_prefix, kv_live_stream)
  *   dgo_merge_partials_f32   closed form m=max m_i, l=sum l_i e^(m_i-m), O=sum O_i e^(m_i-m)/l; the
  *                            reference's state planes: attention_mma_full.metal:107-118,355-368
  *   rounding helpers         src/shaders/common/bf16.rs:9-41, src/shaders/common/f16.rs:3-60
@@ -47,6 +51,8 @@
  *     brute force (lexsort by (-score, index), float64 softmax over the kept set) on random small
  *     cases incl. duplicated keys (tie-break) and ragged causal rows (k > visible keys); the
  *     per-row k rule against hand-computed values
+ *   - FNV-1a: the published test vectors ("" -> offset basis, "a", "foobar"); the snapshot
+ *     restatements: a hand-laid-out two-layer cache, scatter(gather(x)) == x on the live part
  * LSE is not emitted anywhere in the reference; it is the closed form m + ln(l) of the
  * recurrence's own (m, l), cross-checked against a float64 logsumexp of the score row.
  */
@@ -101,6 +107,8 @@ uint32_t dgo_topk_row_k(const uint32_t k_cfg[4], uint32_t n_valid, int causal_ro
 void dgo_attention_topk_f32(const dgo_desc* d, const uint32_t k_cfg[4], const float* q, const float* kv, float* out,
                             uint32_t* sel_idx, uint32_t sel_cap, uint32_t* sel_count, const uint32_t* tok_list,
                             uint32_t n_tok, int n_threads);
+/* FNV-1a over bytes, continuing seed_hash (src/metal/step_kernel/runtime.rs:127-133). */
+uint64_t dgo_fnv1a64(const uint8_t* bytes, size_t n, uint64_t seed_hash);
 /* Same mask semantics, two-pass softmax in double. */
 void dgo_attention_f64(const dgo_desc* d, const float* q, const float* kv, double* out, double* lse,
                        const uint32_t* tok_list, uint32_t n_tok, int n_threads);

@@ -63,6 +63,8 @@ def load():
     lib.dgo_attention_topk_f32.argtypes = [P(Desc), P(C.c_uint32), VP, VP, VP, VP, C.c_uint32, VP, VP, C.c_uint32, C.c_int]
     lib.dgo_topk_row_k.argtypes = [P(C.c_uint32), C.c_uint32, C.c_int]
     lib.dgo_topk_row_k.restype = C.c_uint32
+    lib.dgo_fnv1a64.argtypes = [VP, C.c_size_t, C.c_uint64]
+    lib.dgo_fnv1a64.restype = C.c_uint64
     lib.dgo_attention_blocked_f32.argtypes = [P(Desc), VP, VP, VP, VP, C.c_uint32, C.c_int]
     lib.dgo_attention_partial_f32.argtypes = [P(Desc), VP, VP, C.c_uint32, C.c_uint32, VP, VP, VP, C.c_int]
     lib.dgo_merge_partials_f32.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, VP, VP, VP, VP, VP]
@@ -339,3 +341,57 @@ def synthetic_fill_kv(n, seed):
 
 def max_threads():
     return load().dgo_max_threads()
+
+
+# ---------------------------------------------------------------------------------------
+# KV snapshots and the live-KV fingerprint, on a cache held in the reference's own layout
+# (one byte buffer; per layer a region of `slots` positions, each [K: Hkv*hd | V: Hkv*hd] elements).
+# `layers`: objects with kv_region (byte offset), n_kv_heads, head_dim, slots, kv_ring_mask.
+# ---------------------------------------------------------------------------------------
+
+FNV_OFFSET_BASIS = 0xcbf29ce484222325
+
+
+def fnv1a64(data: bytes, seed_hash: int = FNV_OFFSET_BASIS) -> int:
+    buf = np.frombuffer(bytes(data), dtype=np.uint8)
+    return int(load().dgo_fnv1a64(_ptr(buf) if buf.size else None, buf.size, seed_hash))
+
+
+def _group_bytes(l, elem_bytes):
+    return 2 * l.n_kv_heads * l.head_dim * elem_bytes
+
+
+def kv_gather_prefix(cache: np.ndarray, layers, kv_len: int, elem_bytes: int = 2) -> np.ndarray:
+    """src/metal/step_kv/mod.rs:108-127: per layer the first min(kv_len, slots) slots of the region, concatenated."""
+    out = []
+    for l in layers:
+        n = min(kv_len, l.slots) * _group_bytes(l, elem_bytes)
+        out.append(cache[l.kv_region:l.kv_region + n])
+    return np.concatenate(out) if out else np.zeros(0, np.uint8)
+
+
+def kv_scatter_prefix(cache: np.ndarray, layers, kv_len: int, blob: np.ndarray, elem_bytes: int = 2) -> None:
+    """src/metal/step_kv/mod.rs:133-151: the inverse; bytes past each layer's live prefix stay as they are."""
+    off = 0
+    for l in layers:
+        n = min(kv_len, l.slots) * _group_bytes(l, elem_bytes)
+        cache[l.kv_region:l.kv_region + n] = blob[off:off + n]
+        off += n
+
+
+def kv_live_stream(cache: np.ndarray, layers, kv_len: int, window: int, elem_bytes: int = 2) -> np.ndarray:
+    """The bytes live_kv_fnv eats, in its order (src/metal/step_kernel/runtime.rs:135-147)."""
+    out = []
+    for l in layers:
+        g = _group_bytes(l, elem_bytes)
+        if l.kv_ring_mask == 0:
+            out.append(cache[l.kv_region:l.kv_region + kv_len * g])
+        else:
+            for p in range(max(0, kv_len - window), kv_len):
+                o = l.kv_region + (p & l.kv_ring_mask) * g
+                out.append(cache[o:o + g])
+    return np.concatenate(out) if out else np.zeros(0, np.uint8)
+
+
+def kv_live_fnv(cache: np.ndarray, layers, kv_len: int, window: int, seed_hash: int, elem_bytes: int = 2) -> int:
+    return fnv1a64(kv_live_stream(cache, layers, kv_len, window, elem_bytes).tobytes(), seed_hash)
