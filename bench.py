@@ -377,6 +377,102 @@ def bench_topk(args):
         sys.exit(1)
 
 
+def bench_kv_snapshot(args):
+    """One step = one snapshot of the 30-layer cache at prefix 32768 (gather of every layer's live
+    part into the compact blob) followed by its restore (scatter): byte moves, HBM-bound."""
+    import torch
+    from diffgemma_amd import capi, step_kv
+    from oracle import pyoracle as po
+    kv_len, max_seq = 32768, 32768 + 256
+    layers = step_kv.build_layout(max_seq, capi.DG_BF16, ring_slots=2048)
+    total = step_kv.kv_cache_total_bytes(layers, capi.DG_BF16)
+    arr = step_kv.kv_layers(layers, capi.DG_BF16, "head_major")
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    buf = torch.randint(0, 256, (total,), dtype=torch.uint8, device="cuda", generator=gen)
+    n = step_kv.snapshot_bytes(arr, kv_len)
+    blob = torch.empty(n, dtype=torch.uint8, device="cuda")
+    lib = capi.load()
+    st = torch.cuda.current_stream().cuda_stream
+
+    def gather():
+        capi.check(lib.dg_kv_snapshot_gather(buf.data_ptr(), arr, len(arr), kv_len, blob.data_ptr(), n, st))
+
+    def scatter():
+        capi.check(lib.dg_kv_snapshot_scatter(buf.data_ptr(), arr, len(arr), kv_len, blob.data_ptr(), n, st))
+
+    # check: a few layers against the numpy restatement (the cache re-laid slot-major on the host),
+    # and gather -> scatter into a scrubbed cache -> gather reproduces the blob
+    gather()
+    torch.cuda.synchronize()
+    offs = (C.c_uint64 * len(arr))()
+    tot = C.c_uint64(0)
+    capi.check(lib.dg_kv_snapshot_bytes(arr, len(arr), kv_len, C.byref(tot), offs))
+    ok = True
+    for i in (0, 5, 29):
+        l = layers[i]
+        nb = l.slots * 2 * l.n_kv_heads * l.head_dim * 2
+        reg = buf[l.kv_region:l.kv_region + nb].cpu().numpy().view(np.uint16).reshape(2, l.n_kv_heads, l.slots, l.head_dim)
+        ref_region = np.ascontiguousarray(reg.transpose(2, 0, 1, 3)).view(np.uint8).reshape(-1)     # [slot][K|V][head][d]
+        live = min(kv_len, l.slots) * 2 * l.n_kv_heads * l.head_dim * 2
+        ok = ok and np.array_equal(blob[offs[i]:offs[i] + live].cpu().numpy(), ref_region[:live])
+    keep = blob.clone()
+    buf2 = torch.zeros_like(buf)
+    capi.check(lib.dg_kv_snapshot_scatter(buf2.data_ptr(), arr, len(arr), kv_len, keep.data_ptr(), n, st))
+    capi.check(lib.dg_kv_snapshot_gather(buf2.data_ptr(), arr, len(arr), kv_len, blob.data_ptr(), n, st))
+    torch.cuda.synchronize()
+    ok = ok and torch.equal(blob, keep)
+    t0 = time.perf_counter()
+    h = step_kv.live_kv_fnv(buf, arr, 4096, po.FNV_OFFSET_BASIS, window=1024)
+    t_fnv = time.perf_counter() - t0
+    check = {"bit_exact": bool(ok), "passed": bool(ok), "live_kv_fnv_at_4096": hex(h), "live_kv_fnv_s": t_fnv}
+
+    for _ in range(args.warmup):
+        gather()
+        scatter()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    g_ms = s_ms = 0.0
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ev[0].record()
+        gather()
+        ev[1].record()
+        scatter()
+        ev[2].record()
+        ev[2].synchronize()
+        g_ms += ev[0].elapsed_time(ev[1])
+        s_ms += ev[1].elapsed_time(ev[2])
+    t1 = time.perf_counter()
+    g_ms /= args.steps
+    s_ms /= args.steps
+    ms = (t1 - t0) * 1e3 / args.steps
+    moved = 2.0 * n                    # every live byte is read once and written once, per direction
+    res = {"metric": "KV snapshot + restore of the 30-layer cache @ 32k prefix: GB/s moved (read + write), 1 GPU",
+           "value": 2 * moved / ((g_ms + s_ms) * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "u8", "data": "synthetic",
+           "config": {"workload": "kv_snapshot", "layers": len(layers), "kv_prefix": kv_len, "cache_bytes": total,
+                      "snapshot_bytes": n, "cache_layout": "bf16 head-major planes, sliding layers rings of 2048 slots"},
+           "kernels": {"gather_ms": g_ms, "scatter_ms": s_ms},
+           "roofline": {"bound": "hbm", "achieved": moved / (min(g_ms, s_ms) * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": moved / (min(g_ms, s_ms) * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "kernel": "kv_move_kernel", "kernel_ms": min(g_ms, s_ms)},
+           "check": check}
+    if not args.no_cpu_baseline:
+        # the reference's own form of the gather: slices of a host buffer concatenated (numpy memcpy)
+        host = np.zeros(total, np.uint8)
+        t0 = time.perf_counter()
+        ref_blob = po.kv_gather_prefix(host, layers, kv_len)
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": 2.0 * ref_blob.size / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"one gather of the whole snapshot ({ref_blob.size} bytes) from a host buffer in the "
+                                         f"reference's layout, {dt:.2f} s, numpy slice copies"}
+    print(json.dumps(res), flush=True)
+    if not check["passed"]:
+        sys.exit(1)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -410,6 +506,9 @@ def main():
         return
     if args.workload in TOPK_SHAPES:
         bench_topk(args)
+        return
+    if args.workload == "kv_snapshot":
+        bench_kv_snapshot(args)
         return
 
     w = W.config(args.workload)
