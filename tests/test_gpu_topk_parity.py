@@ -163,6 +163,28 @@ def test_global_layer_at_32k_prefix_rows(gpu_ready, po):
     assert max_abs_diff(got[toks], ref[toks]) <= 2e-2 and mean_abs_diff(got[toks], ref[toks]) <= 2e-3
 
 
+def test_long_context_rows(gpu_ready, po):
+    """131072-key prefix with 1% of the keys scaled x8 (config 4's inputs): k = 512 (the cap), score rows of
+    525 KB, sixteen blocks of canvas rows."""
+    import torch
+    w = W.config("cfg4_long")
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+    d = w.desc()
+    d.out_dtype = capi.DG_F32
+    k_cfg = T.adaptive_k()
+    out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.float32, device="cuda")
+    T.forward(d, k_cfg, qd, kd, out, T.alloc_workspace(d, k_cfg))
+    torch.cuda.synchronize()
+    toks = np.array([0, 17, 128, 255], dtype=np.uint32)
+    od = po.make_desc(w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, layout=w.layout, t_cap=w.t_all)
+    ref, idx, cnt = po.attention_topk_f32(od, k_cfg, q, kv, tok_list=toks, sel_cap=512)
+    assert (cnt[toks] == 512).all()
+    got = out.cpu().numpy().reshape(w.canvas, w.n_q_heads, w.head_dim)
+    assert np.isfinite(got).all()
+    assert max_abs_diff(got[toks], ref[toks]) <= 2e-2 and mean_abs_diff(got[toks], ref[toks]) <= 2e-3
+
+
 # ------------------------------------------------------------------ edge cases
 EDGE = [
     # canvas, hq, hkv, hd, kv_len, causal_rows, window, k_cfg
