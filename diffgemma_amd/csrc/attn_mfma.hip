@@ -616,16 +616,29 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     const uint32_t rbk = rgrp * NRBW + j;
     const uint32_t rr = row0 + rbk * 32u + l32;
     if (p.n_splits > 1) {
-      const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + rr;
+      // The accumulators hold a row per lane: stored as they are, every instruction would
+      // scatter 32-byte pieces over 32 rows.  Each wave passes its 32 rows x (NDBW x 32) d through
+      // its own piece of LDS (the tile buffers are free now) and writes whole rows instead.
+      constexpr int STG_ROW = NDBW * 128 + 16;            // bytes; the pad keeps the 16-byte writes of 8 rows apart
+      constexpr int LPR = NDBW * 8, RPI = 64 / LPR;       // lanes per row slice, rows per store instruction
+      static_assert(4 * 32 * STG_ROW <= OFF_ML, "staging must not reach the (m, l) words");
+      lds_char* const stg = (lds_char*)smem + wave * (32 * STG_ROW);
 #pragma unroll
       for (int i = 0; i < NDBW; ++i) {
-        float* po = p.part_o + prow * D + 32u * (dgrp * NDBW + i) + 4u * g2;
+        const f32x16& a = o[i * NRBW + j];
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
-          const f32x16& a = o[i * NRBW + j];
           f32x4 v4 = {a[4 * q4], a[4 * q4 + 1], a[4 * q4 + 2], a[4 * q4 + 3]};
-          *(f32x4*)(po + 8 * q4) = v4;
+          *(__attribute__((address_space(3))) f32x4*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 4) = v4;
         }
+      }
+      const size_t prow0 = ((size_t)split * p.hkv + kvh) * p.rows_pad + row0 + rbk * 32u;
+      float* const po = p.part_o + prow0 * D + 32u * (dgrp * NDBW) + (lane % LPR) * 4u;
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const uint32_t rl = it * RPI + lane / LPR;        // row within the block
+        const f32x4 v4 = *(__attribute__((address_space(3))) f32x4*)(stg + rl * STG_ROW + (lane % LPR) * 16);
+        *(f32x4*)(po + (size_t)rl * D) = v4;
       }
       continue;
     }
