@@ -149,6 +149,12 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
     }
     if (p.out_dtype == DT_F32) {
       ((float4*)((float*)p.out + ooff))[d4] = o;
+    } else if (p.out_dtype == DT_BF16) {   // four bf16 in one 8-byte store
+      const bool tr = p.out_trunc != 0;
+      uint2 pk;
+      pk.x = (uint32_t)f32_to_bf16_bits(o.x, tr) | ((uint32_t)f32_to_bf16_bits(o.y, tr) << 16);
+      pk.y = (uint32_t)f32_to_bf16_bits(o.z, tr) | ((uint32_t)f32_to_bf16_bits(o.w, tr) << 16);
+      ((uint2*)((uint16_t*)p.out + ooff))[d4] = pk;
     } else {
       store_out(p, ooff + d4 * 4 + 0, o.x);
       store_out(p, ooff + d4 * 4 + 1, o.y);
