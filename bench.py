@@ -608,17 +608,24 @@ def main():
         check["passed"] = bool(check["passed"] and check["timed_steps_reproduce_checked_output"])
 
     # ---- what nothing but MFMAs sustains on this machine, right after the timed steps ----
+    # Two operand sets: near-constant values (little multiplier power, the clock stays high) and
+    # random sign/exponent/mantissa, which is what attention feeds the matrix cores.  Each figure
+    # is the rate of about 20 ms of back-to-back launches, after a pass that warms the code up.
     lib = capi.load()
     sink = torch.zeros(256 * 256, dtype=torch.float32, device="cuda")
     mf = C.c_uint64(0)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for rep in range(2):                   # first pass warms the code up
-        e0.record()
-        for _ in range(8):
-            capi.check(lib.dg_calib_mfma(sink.data_ptr(), sink.numel() * 4, 256, 1000, C.byref(mf), A.stream_handle()))
-        e1.record()
-        torch.cuda.synchronize()
-    mfma_only_tflops = 8 * mf.value / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    mfma_only = {}
+    for random_operands in (0, 1):
+        for rep in range(2):
+            e0.record()
+            for _ in range(8):
+                capi.check(lib.dg_calib_mfma(sink.data_ptr(), sink.numel() * 4, 256, 8000, random_operands,
+                                             C.byref(mf), A.stream_handle()))
+            e1.record()
+            torch.cuda.synchronize()
+        mfma_only[random_operands] = 8 * mf.value / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    mfma_only_tflops, mfma_random_tflops = mfma_only[0], mfma_only[1]
 
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kern_tflops = flops / (kern_ms * 1e-3) / 1e12
@@ -646,6 +653,8 @@ def main():
                      "kernel": "attn_mfma_kernel", "kernel_ms": kern_ms,
                      "mfma_only_microkernel_tflops": mfma_only_tflops,
                      "frac_of_mfma_only_microkernel": kern_tflops / mfma_only_tflops,
+                     "mfma_only_random_operands_tflops": mfma_random_tflops,
+                     "frac_of_mfma_only_random_operands": kern_tflops / mfma_random_tflops,
                      "kv_gbs": kv_bytes / (kern_ms * 1e-3) / 1e9, "hbm_peak_gbs": PEAK_HBM_GBS},
         "rounds": rounds, "check": check, "input_gen_s": t_gen,
     }

@@ -153,7 +153,7 @@ def load():
     lib.dg_layer_kv_slots.restype = C.c_uint64
     lib.dg_calib_copy.argtypes = [VP, VP, C.c_size_t, VP]
     lib.dg_calib_copy.restype = C.c_int
-    lib.dg_calib_mfma.argtypes = [VP, C.c_size_t, C.c_uint32, C.c_uint32, P(C.c_uint64), VP]
+    lib.dg_calib_mfma.argtypes = [VP, C.c_size_t, C.c_uint32, C.c_uint32, C.c_uint32, P(C.c_uint64), VP]
     lib.dg_calib_mfma.restype = C.c_int
     lib.dg_qk_rope_kv.argtypes = [P(RopeDesc), VP, VP, VP, VP, VP, VP, VP, VP]
     lib.dg_qk_rope_kv.restype = C.c_int

@@ -205,26 +205,48 @@ __global__ void calib_copy_kernel(const uint4* __restrict__ src, uint4* __restri
 
 // Nothing but MFMAs: four independent 32x32x16 bf16 accumulators per wave, one wave per SIMD.
 // What this sustains is the ceiling the attention kernel's MFMA rate is compared with on the
-// machine at hand (the published peak assumes the maximum clock).
+// machine at hand.  The published peak assumes the maximum clock; the clock the chip holds
+// depends on the power the multipliers draw, which depends on the operand values: with
+// RANDOM operands (eight fragments per side of sign/exponent/mantissa noise around unit
+// magnitude, cycled) the same instruction stream runs at a clearly lower clock than with the
+// near-constant ones.
 typedef float calib_f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 calib_bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t calib_u32x4 __attribute__((ext_vector_type(4)));
+template <bool RANDOM>
 __global__ void __launch_bounds__(256) calib_mfma_kernel(float* sink, uint32_t iters) {
-  calib_bf16x8 a, b;
+  calib_u32x4 a[8], b[8];
+  uint32_t seed = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+  auto noise_pair = [&]() -> uint32_t {   // two bf16 of random sign, magnitude in [2^-7, 2)
+    seed ^= seed << 13;
+    seed ^= seed >> 17;
+    seed ^= seed << 5;
+    const uint32_t lo = ((seed & 1u) << 15) | ((120u + ((seed >> 1) & 7u)) << 7) | ((seed >> 4) & 0x7fu);
+    const uint32_t hi = (((seed >> 11) & 1u) << 15) | ((120u + ((seed >> 12) & 7u)) << 7) | ((seed >> 15) & 0x7fu);
+    return lo | (hi << 16);
+  };
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    a[i] = (__bf16)(1.0f + 0.001f * (float)((threadIdx.x + i) & 7));
-    b[i] = (__bf16)(0.5f - 0.001f * (float)((threadIdx.x * 3 + i) & 7));
-  }
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // near-constant: 1 + k/128 and 1/2 - k/256 for small k (a few mantissa bits set)
+      a[i][e] = RANDOM ? noise_pair() : 0x3f803f80u + ((threadIdx.x + e) & 3u);
+      b[i][e] = RANDOM ? noise_pair() : 0x3f003f00u - ((threadIdx.x * 3u + e) & 3u);
+    }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(a[i]), "+v"(b[i]));   // keep sixteen distinct fragments
   calib_f32x16 c0, c1, c2, c3;
 #pragma unroll
   for (int e = 0; e < 16; ++e) c0[e] = c1[e] = c2[e] = c3[e] = 0.f;
+  auto fa = [&](int i) { return __builtin_bit_cast(calib_bf16x8, a[i & 7]); };
+  auto fb = [&](int i) { return __builtin_bit_cast(calib_bf16x8, b[(i * 3) & 7]); };
   for (uint32_t it = 0; it < iters; ++it) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
-      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
-      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
-      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa(4 * u), fb(4 * u), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa(4 * u + 1), fb(4 * u + 1), c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa(4 * u + 2), fb(4 * u + 2), c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa(4 * u + 3), fb(4 * u + 3), c3, 0, 0, 0);
     }
   }
   float acc = 0.f;
@@ -235,8 +257,9 @@ __global__ void __launch_bounds__(256) calib_mfma_kernel(float* sink, uint32_t i
 
 }  // namespace
 
-hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, hipStream_t s) {
-  hipLaunchKernelGGL(calib_mfma_kernel, dim3(workgroups), dim3(256), 0, s, sink, iters);
+hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, bool random_operands, hipStream_t s) {
+  if (random_operands) hipLaunchKernelGGL(calib_mfma_kernel<true>, dim3(workgroups), dim3(256), 0, s, sink, iters);
+  else hipLaunchKernelGGL(calib_mfma_kernel<false>, dim3(workgroups), dim3(256), 0, s, sink, iters);
   return hipGetLastError();
 }
 

@@ -257,9 +257,12 @@ int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream);
  * `*flops` = the floating-point operations it performs; the caller times it.  `sink` (at
  * least workgroups*256 floats, device memory) is never written in practice.  What this
  * sustains is the MFMA ceiling of the machine at hand, next to which the attention kernel's
- * rate is read.  Measurement aid, no counterpart in the reference. */
-int dg_calib_mfma(float* sink, size_t sink_bytes, uint32_t workgroups, uint32_t iters, uint64_t* flops,
-                  void* stream);
+ * rate is read.  `random_operands` = 0: near-constant operands (the multipliers draw little
+ * power and the clock stays high); 1: operands of random sign, exponent and mantissa, which
+ * is what attention feeds the matrix cores (the clock the chip then holds is lower).
+ * Measurement aid, no counterpart in the reference. */
+int dg_calib_mfma(float* sink, size_t sink_bytes, uint32_t workgroups, uint32_t iters, uint32_t random_operands,
+                  uint64_t* flops, void* stream);
 
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);
