@@ -13,6 +13,7 @@ DG_KERNEL_AUTO, DG_KERNEL_SCALAR, DG_KERNEL_MFMA = 0, 1, 2
 DG_ATTN_F_OUT_TRUNCATE = 0x1
 DG_ATTN_F_CAUSAL_SEES_MASKED = 0x2
 DG_ATTN_F_T_LO_EXPLICIT = 0x4
+DG_ATTN_F_F32_PARTIALS = 0x8
 
 DG_ROPE_F_QK_TRUNCATE = 0x1
 

@@ -122,9 +122,67 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
   const float inv = den > 0.f ? 1.f / den : 0.f;
   const float w_mine = ls > 0.f ? exp2f(ms - mx) * inv : 0.f;   // weight of split `lane`
   const size_t ooff = ((size_t)tok * p.hq + qh) * hd;
-  const float* const base = p.part_o + row * hd;
   const size_t sstride = split_stride * hd;
-  for (uint32_t d4 = lane; d4 < hd / 4; d4 += 64) {
+  if (p.part_half) {
+    // normalised f16 partial rows: O = sum_s (l_s 2^(m_s - m) / den) O_s; eight d per lane and load
+    const float w_half = wl * inv;
+    const uint16_t* const hbase = (const uint16_t*)p.part_o + row * hd;
+    // (every lane runs the loop, idle ones on chunk 0: the weight shuffles below read lanes
+    // that would otherwise be switched off when head_dim / 8 is below the split count)
+    for (uint32_t d8_0 = 0; d8_0 < hd / 8; d8_0 += 64) {
+      const bool live = d8_0 + lane < hd / 8;
+      const uint32_t d8 = live ? d8_0 + lane : 0u;
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      uint32_t s = 0;
+      for (; s + 4 <= p.n_splits; s += 4) {
+        uint4 a[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a[u] = ((const uint4*)(hbase + (s + u) * sstride))[d8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float w = __shfl(w_half, s + u, 64);
+          const uint32_t wd[4] = {a[u].x, a[u].y, a[u].z, a[u].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            acc[2 * e] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] & 0xffffu));
+            acc[2 * e + 1] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] >> 16));
+          }
+        }
+      }
+      for (; s < p.n_splits; ++s) {
+        const uint4 a = ((const uint4*)(hbase + s * sstride))[d8];
+        const float w = __shfl(w_half, s, 64);
+        const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[2 * e] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] & 0xffffu));
+          acc[2 * e + 1] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] >> 16));
+        }
+      }
+      if (!live) continue;
+      if (p.out_dtype == DT_BF16) {   // eight bf16 in one 16-byte store
+        const bool tr = p.out_trunc != 0;
+        uint4 pk;
+        pk.x = (uint32_t)f32_to_bf16_bits(acc[0], tr) | ((uint32_t)f32_to_bf16_bits(acc[1], tr) << 16);
+        pk.y = (uint32_t)f32_to_bf16_bits(acc[2], tr) | ((uint32_t)f32_to_bf16_bits(acc[3], tr) << 16);
+        pk.z = (uint32_t)f32_to_bf16_bits(acc[4], tr) | ((uint32_t)f32_to_bf16_bits(acc[5], tr) << 16);
+        pk.w = (uint32_t)f32_to_bf16_bits(acc[6], tr) | ((uint32_t)f32_to_bf16_bits(acc[7], tr) << 16);
+        ((uint4*)((uint16_t*)p.out + ooff))[d8] = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) store_out(p, ooff + d8 * 8 + e, acc[e]);
+      }
+    }
+    if (lane == 0) {
+      if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));
+      if (p.lse) p.lse[(size_t)tok * p.hq + qh] = den > 0.f ? mx * kLn2 + logf(den) : -INFINITY;
+    }
+    return;
+  }
+  const float* const base = p.part_o + row * hd;
+  for (uint32_t d4_0 = 0; d4_0 < hd / 4; d4_0 += 64) {   // idle lanes run along, see above
+    const bool live = d4_0 + lane < hd / 4;
+    const uint32_t d4 = live ? d4_0 + lane : 0u;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     uint32_t s = 0;
     for (; s + 4 <= p.n_splits; s += 4) {
@@ -147,6 +205,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
       o.z += w * a.z;
       o.w += w * a.w;
     }
+    if (!live) continue;
     if (p.out_dtype == DT_F32) {
       ((float4*)((float*)p.out + ooff))[d4] = o;
     } else if (p.out_dtype == DT_BF16) {   // four bf16 in one 8-byte store

@@ -615,6 +615,36 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   for (int j = 0; j < NRBW; ++j) {
     const uint32_t rbk = rgrp * NRBW + j;
     const uint32_t rr = row0 + rbk * 32u + l32;
+    if (p.n_splits > 1 && p.part_half) {
+      // Same route through LDS as below, for partial rows kept as f16: each accumulator is divided
+      // by the split's row sum first (a weighted mean of V rows: no larger than the largest |V|),
+      // and the merge weighs the rows by l 2^(m - m_max) instead of 2^(m - m_max).
+      constexpr int STG_ROW = NDBW * 64 + 16;             // bytes of a staged row slice, padded
+      constexpr int LPR = NDBW * 4, RPI = 64 / LPR;       // lanes per row slice (16 B each), rows per store
+      lds_char* const stg = (lds_char*)smem + wave * (32 * STG_ROW);
+      const float l_row = sml[(rbk * 32u + l32) * 2u + 1u];
+      const float inv = l_row > 0.f ? 1.f / l_row : 0.f;
+#pragma unroll
+      for (int i = 0; i < NDBW; ++i) {
+        const f32x16& a = o[i * NRBW + j];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          u32x2 h2;
+          h2[0] = pack2<true>(a[4 * q4] * inv, a[4 * q4 + 1] * inv);
+          h2[1] = pack2<true>(a[4 * q4 + 2] * inv, a[4 * q4 + 3] * inv);
+          *(__attribute__((address_space(3))) u32x2*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 2) = h2;
+        }
+      }
+      const size_t prow0 = ((size_t)split * p.hkv + kvh) * p.rows_pad + row0 + rbk * 32u;
+      uint16_t* const po = (uint16_t*)p.part_o + prow0 * D + 32u * (dgrp * NDBW) + (lane % LPR) * 8u;
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const uint32_t rl = it * RPI + lane / LPR;        // row within the block
+        const u32x4 v4 = *(lds_u32x4*)(stg + rl * STG_ROW + (lane % LPR) * 16);
+        *(u32x4*)(po + (size_t)rl * D) = v4;
+      }
+      continue;
+    }
     if (p.n_splits > 1) {
       // The accumulators hold a row per lane: stored as they are, every instruction would
       // scatter 32-byte pieces over 32 rows.  Each wave passes its 32 rows x (NDBW x 32) d through

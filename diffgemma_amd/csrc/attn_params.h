@@ -22,7 +22,8 @@ struct AttnParams {
   const void* v;       // layer region + V offset
   void* out;           // [canvas][hq][D]
   float* lse;          // [canvas][hq] or null
-  float* part_o;       // [split][hkv][rows_pad][D] unnormalised accumulators
+  float* part_o;       // [split][hkv][rows_pad][D]: unnormalised fp32 accumulators, or (part_half) the same
+                       // index space in f16 holding accumulators divided by the split's row sum
   float* part_ml;      // [split][hkv][rows_pad][2] (m in log2 units, l)
   uint32_t* dbg;       // 4 words, first-writer-wins, or null
   unsigned long long* phase_cycles;  // [workgroup][wave][8] cycle sums; only written by builds with DG_ATTN_PHASE_TIMING
@@ -38,6 +39,7 @@ struct AttnParams {
   uint32_t n_splits, tile_first, tiles_per_split, tile_end;
   uint32_t q_is_bf16;    // Q holds bf16 although E is f16 (reference: bf16 activations, f16 cache)
   uint32_t out_dtype, out_trunc;
+  uint32_t part_half;    // split partials are normalised f16 rows instead of unnormalised fp32 ones
   float scale_log2;      // softmax_scale * log2(e)
 };
 

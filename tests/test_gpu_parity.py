@@ -171,6 +171,26 @@ def test_split_count_invariance_full_size(gpu_ready):
         assert np.max(np.abs(lse - base_lse) / np.abs(base_lse)) < 1e-4, s
 
 
+@pytest.mark.parametrize("hd,hq,hkv,splits", [(32, 8, 4, 17), (64, 32, 4, 9), (128, 8, 4, 33), (256, 16, 8, 8), (256, 16, 8, 64)])
+def test_split_partial_formats(gpu_ready, po, hd, hq, hkv, splits):
+    """Split partial rows travel as normalised f16 rows by default at head_dim <= 256 with a 16-bit output
+    (DG_ATTN_F_F32_PARTIALS keeps fp32): both formats meet the oracle, they differ by output roundings
+    only, and an f32 output keeps fp32 partials.  The split counts are larger than head_dim / 8 and
+    head_dim / 4: the merge reads every split's weight whatever lanes its loads keep busy."""
+    w = W.Workload("partials", 100, hq, hkv, hd, 2049, causal_rows=50, seed=11)
+    half = run_workload(po, w, n_splits=splits)
+    full = run_workload(po, w, n_splits=splits, flags=capi.DG_ATTN_F_F32_PARTIALS)
+    check_tolerances(*half)
+    check_tolerances(*full)
+    diff = np.abs(half[0] - full[0])
+    assert diff.max() <= 2.0 ** -7 * max(1.0, np.abs(full[0]).max())       # one bf16 step of the largest value
+    assert np.mean(diff > 0) < 0.1                                         # and only where a rounding tipped
+    assert np.max(np.abs(half[1] - full[1])) == 0.0                        # (m, l) travel in fp32 either way
+    f32a = run_workload(po, w, n_splits=splits, out_f32=True)
+    f32b = run_workload(po, w, n_splits=splits, out_f32=True, flags=capi.DG_ATTN_F_F32_PARTIALS)
+    assert np.array_equal(f32a[0], f32b[0])
+
+
 def test_scalar_and_mfma_kernels_agree_full_size(gpu_ready):
     w = W.scaled(W.config("cfg3_global"), 8192)
     q, kv = W.generate(w)
