@@ -46,6 +46,19 @@ namespace {
 // log2 units by which a tile max may exceed the reference max before the reference is raised
 template <bool F16>
 constexpr float kTau = F16 ? 15.0f : 80.0f;
+// The probabilities are stored as 2^(score - reference - kPOff): with bf16 the offset moves
+// their range to [2^-126, 2^-6], so that a key whose weight is below 2^-40 of the reference
+// (and therefore of the row's largest) underflows to an exact zero in the exponential itself.
+// Dropping those weights changes a row's sum by less than keys x 2^-40, far below the fp32
+// rounding of the accumulation; what it buys is power: most keys of a long row are that
+// small, a multiplier fed zeros draws little, and the clock of this kernel is set by the power
+// of the matrix cores.  (f16 probabilities already underflow below 2^-25.)
+template <bool F16>
+constexpr float kPOff = F16 ? 0.0f : 86.0f;
+// The reference lags the row's running max by up to kTau, so on top of that a weight is dropped
+// (set to an exact zero) when its score is more than kDrop below the running max itself: the
+// same bound on the error, and on a long row all but a fraction of a per cent of the keys.
+constexpr float kDrop = 40.0f;
 
 // Optional per-phase cycle accounting (development builds only): every wave sums the cycles
 // it spends in each phase of the tile loop and stores the sums at the end.
@@ -272,6 +285,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[i][e] = 0.f;
   float m_ref = -INFINITY;  // running reference max, log2 units (scale folded in)
+  float m_run = -INFINITY;  // running max itself
+  float s_drop = -INFINITY; // raw scores below this are dropped (tracks m_run)
+  const float inv_scale_log2 = 1.f / p.scale_log2;
   float l_part = 0.f;       // this lane's share of the row sum (its 16 of every 32 keys),
   float l_part2 = 0.f;      // kept as two partial sums
 
@@ -386,7 +402,11 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           m_ref = m_new;
         }
         if (lane == 0) ((uint32_t*)(smem + OFF_FLAG + par * FLAG_BYTES))[wave] = rescale ? 1u : 0u;
-        m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+        m_use = (m_ref == -INFINITY) ? 0.f : m_ref + kPOff<F16>;
+        if constexpr (!F16) {
+          m_run = fmaxf(m_run, tmax);
+          s_drop = (m_run - kDrop) * inv_scale_log2;
+        }
       } else {
         // scores 4 q .. 4 q + 3 in two steps: (a) scale and subtract, first two exponentials;
         // (b) the other two exponentials, rounding to the MFMA operand type, and for every
@@ -397,9 +417,17 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           for (int i = 0; i < 4; ++i) ex[i] = __builtin_fmaf(s[4 * q + i], p.scale_log2, -m_use);
           ex[0] = __builtin_amdgcn_exp2f(ex[0]);
           ex[1] = __builtin_amdgcn_exp2f(ex[1]);
+          if constexpr (!F16) {
+            ex[0] = s[4 * q + 0] >= s_drop ? ex[0] : 0.f;
+            ex[1] = s[4 * q + 1] >= s_drop ? ex[1] : 0.f;
+          }
         } else {
           ex[2] = __builtin_amdgcn_exp2f(ex[2]);
           ex[3] = __builtin_amdgcn_exp2f(ex[3]);
+          if constexpr (!F16) {
+            ex[2] = s[4 * q + 2] >= s_drop ? ex[2] : 0.f;
+            ex[3] = s[4 * q + 3] >= s_drop ? ex[3] : 0.f;
+          }
           pk4[(2 * q) % 4] = pack2<F16>(ex[0], ex[1]);
           pk4[(2 * q + 1) % 4] = pack2<F16>(ex[2], ex[3]);
           if constexpr (q % 2 == 1) {
@@ -597,16 +625,17 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   DG_PHASE_STORE
   // row owners publish (m, l) of their rows; d owners normalise and store their slice of O
   const float l_tot = sum_across_halves(l_part + l_part2);
+  const float m_pub = m_ref + kPOff<F16>;   // the exponent the sums are relative to
   __syncthreads();   // the last tile's readers are done with LDS
   if (g2 == 0) {
-    sml[(wave * 32u + l32) * 2u] = m_ref;
+    sml[(wave * 32u + l32) * 2u] = m_pub;
     sml[(wave * 32u + l32) * 2u + 1u] = l_tot;
     if (p.n_splits > 1) {
       const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + r;
-      p.part_ml[prow * 2] = m_ref;
+      p.part_ml[prow * 2] = m_pub;
       p.part_ml[prow * 2 + 1] = l_tot;
     } else if (row_ok) {
-      if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l_tot > 0.f ? m_ref * kLn2 + __logf(l_tot) : -INFINITY;
+      if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l_tot > 0.f ? m_pub * kLn2 + __logf(l_tot) : -INFINITY;
       if (p.dbg && !(l_tot > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l_tot));
     }
   }
