@@ -286,8 +286,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     for (int e = 0; e < 16; ++e) o[i][e] = 0.f;
   float m_ref = -INFINITY;  // running reference max, log2 units (scale folded in)
   float m_run = -INFINITY;  // running max itself
-  float s_drop = -INFINITY; // raw scores below this are dropped (tracks m_run)
-  const float inv_scale_log2 = 1.f / p.scale_log2;
+  float x_drop = -INFINITY; // exponents below this are dropped: m_run - kDrop, relative to the reference in use
   float l_part = 0.f;       // this lane's share of the row sum (its 16 of every 32 keys),
   float l_part2 = 0.f;      // kept as two partial sums
 
@@ -405,7 +404,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         m_use = (m_ref == -INFINITY) ? 0.f : m_ref + kPOff<F16>;
         if constexpr (!F16) {
           m_run = fmaxf(m_run, tmax);
-          s_drop = (m_run - kDrop) * inv_scale_log2;
+          x_drop = m_run - kDrop - m_use;
         }
       } else {
         // scores 4 q .. 4 q + 3 in two steps: (a) scale and subtract, first two exponentials;
@@ -415,19 +414,17 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         if constexpr ((c - 3) % 2 == 0) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) ex[i] = __builtin_fmaf(s[4 * q + i], p.scale_log2, -m_use);
+          const bool keep0 = F16 || ex[0] >= x_drop, keep1 = F16 || ex[1] >= x_drop;
           ex[0] = __builtin_amdgcn_exp2f(ex[0]);
           ex[1] = __builtin_amdgcn_exp2f(ex[1]);
-          if constexpr (!F16) {
-            ex[0] = s[4 * q + 0] >= s_drop ? ex[0] : 0.f;
-            ex[1] = s[4 * q + 1] >= s_drop ? ex[1] : 0.f;
-          }
+          ex[0] = keep0 ? ex[0] : 0.f;
+          ex[1] = keep1 ? ex[1] : 0.f;
         } else {
+          const bool keep2 = F16 || ex[2] >= x_drop, keep3 = F16 || ex[3] >= x_drop;
           ex[2] = __builtin_amdgcn_exp2f(ex[2]);
           ex[3] = __builtin_amdgcn_exp2f(ex[3]);
-          if constexpr (!F16) {
-            ex[2] = s[4 * q + 2] >= s_drop ? ex[2] : 0.f;
-            ex[3] = s[4 * q + 3] >= s_drop ? ex[3] : 0.f;
-          }
+          ex[2] = keep2 ? ex[2] : 0.f;
+          ex[3] = keep3 ? ex[3] : 0.f;
           pk4[(2 * q) % 4] = pack2<F16>(ex[0], ex[1]);
           pk4[(2 * q + 1) % 4] = pack2<F16>(ex[2], ex[3]);
           if constexpr (q % 2 == 1) {
