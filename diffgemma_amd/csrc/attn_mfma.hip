@@ -44,20 +44,21 @@ namespace dg {
 namespace {
 
 // log2 units by which a tile max may exceed the reference max before the reference is raised
+// (a raise rescales a 32-row block of O, which costs about as much as a tile's P.V).  With the
+// offset below the bf16 probabilities then reach 2^34 at most, and a row's sums 2^34 x keys x |v|.
 template <bool F16>
-constexpr float kTau = F16 ? 15.0f : 80.0f;
+constexpr float kTau = F16 ? 15.0f : 120.0f;
 // The probabilities are stored as 2^(score - reference - kPOff): with bf16 the offset moves
-// their range to [2^-126, 2^-6], so that a key whose weight is below 2^-40 of the reference
+// their range to [2^-126, 2^34], so that a key whose weight is below 2^-40 of the reference
 // (and therefore of the row's largest) underflows to an exact zero in the exponential itself.
-// Dropping those weights changes a row's sum by less than keys x 2^-40, far below the fp32
-// rounding of the accumulation; what it buys is power: most keys of a long row are that
-// small, a multiplier fed zeros draws little, and the clock of this kernel is set by the power
-// of the matrix cores.  (f16 probabilities already underflow below 2^-25.)
+// The reference lags the row's running max by up to kTau, so on top of that a weight is set to
+// an exact zero when its score is more than kDrop below the running max.  Dropping those
+// weights changes a row's sum by less than keys x 2^-40 of it, below the fp32 rounding of the
+// accumulation; what it buys is power: on a long row all but a per cent or two of the keys are
+// that small, a multiplier fed zeros draws little, and the clock this kernel runs at is set by
+// the power of the matrix cores.  (f16 probabilities already underflow 2^-25 below 2^15.)
 template <bool F16>
 constexpr float kPOff = F16 ? 0.0f : 86.0f;
-// The reference lags the row's running max by up to kTau, so on top of that a weight is dropped
-// (set to an exact zero) when its score is more than kDrop below the running max itself: the
-// same bound on the error, and on a long row all but a fraction of a per cent of the keys.
 constexpr float kDrop = 40.0f;
 
 // Optional per-phase cycle accounting (development builds only): every wave sums the cycles
