@@ -325,7 +325,7 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   p.q_is_bf16 = pl.q_is_bf16 ? 1u : 0u;
   p.out_dtype = d->out_dtype;
   p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
-  p.part_half = (pl.n_splits > 1 && d->head_dim <= 256 && d->out_dtype != DG_F32 && !(d->flags & DG_ATTN_F_F32_PARTIALS))
+  p.part_half = (pl.n_splits > 1 && d->out_dtype != DG_F32 && !(d->flags & DG_ATTN_F_F32_PARTIALS))
                     ? 1u
                     : 0u;
   p.scale_log2 = pl.scale * dg::kLog2e;

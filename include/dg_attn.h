@@ -61,13 +61,13 @@ typedef enum dg_kernel_sel {
 #define DG_ATTN_F_CAUSAL_SEES_MASKED 0x2u  /* causal rows also see canvas keys >= kv_len+causal_rows */
 #define DG_ATTN_F_T_LO_EXPLICIT 0x4u       /* non-causal rows start at desc.t_lo instead of the
                                               window rule kv_len-(window-1) */
-#define DG_ATTN_F_F32_PARTIALS 0x8u        /* keep split partial rows in fp32.  Default for head_dim <= 256
-                                              with a 16-bit output: partial rows travel between the
-                                              attention and the merge kernel as f16 after division by
-                                              the split's row sum (a weighted mean of V rows, so it
-                                              needs |V| <= 65504, which an f16 cache guarantees; the
-                                              rounding is 1/8 of the output's).  head_dim 512 and f32
-                                              outputs always use fp32 partials. */
+#define DG_ATTN_F_F32_PARTIALS 0x8u        /* keep split partial rows in fp32.  Default with a 16-bit
+                                              output: partial rows travel between the attention and
+                                              the merge kernel as f16 after division by the split's
+                                              row sum (a weighted mean of V rows, so it needs
+                                              |V| <= 65504, which an f16 cache guarantees; the
+                                              rounding is 1/8 of the output's).  f32 outputs always
+                                              use fp32 partials. */
 
 typedef struct dg_attn_desc {
   uint32_t canvas;        /* query rows; the reference passes active_canvas (256/128/64) */

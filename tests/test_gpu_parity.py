@@ -171,9 +171,10 @@ def test_split_count_invariance_full_size(gpu_ready):
         assert np.max(np.abs(lse - base_lse) / np.abs(base_lse)) < 1e-4, s
 
 
-@pytest.mark.parametrize("hd,hq,hkv,splits", [(32, 8, 4, 17), (64, 32, 4, 9), (128, 8, 4, 33), (256, 16, 8, 8), (256, 16, 8, 64)])
+@pytest.mark.parametrize("hd,hq,hkv,splits", [(32, 8, 4, 17), (64, 32, 4, 9), (128, 8, 4, 33), (256, 16, 8, 8), (256, 16, 8, 64),
+                                              (512, 16, 2, 8), (512, 8, 1, 40)])
 def test_split_partial_formats(gpu_ready, po, hd, hq, hkv, splits):
-    """Split partial rows travel as normalised f16 rows by default at head_dim <= 256 with a 16-bit output
+    """Split partial rows travel as normalised f16 rows by default with a 16-bit output
     (DG_ATTN_F_F32_PARTIALS keeps fp32): both formats meet the oracle, they differ by output roundings
     only, and an f32 output keeps fp32 partials.  The split counts are larger than head_dim / 8 and
     head_dim / 4: the merge reads every split's weight whatever lanes its loads keep busy."""
@@ -324,13 +325,18 @@ def test_truncating_store_matches_reference_rounding(gpu_ready):
     import torch
     f = A.model_full_fixture(300, canvas=32)
     rig = A.AttnRig.from_fixture(f)
-    d32 = rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=False)
+
+    def desc(truncate):   # the same fp32 partial rows behind all three stores
+        d = rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=truncate)
+        d.flags |= capi.DG_ATTN_F_F32_PARTIALS
+        return d
+    d32 = desc(False)
     d32.out_dtype = capi.DG_F32
     out32 = torch.zeros(f.out_len(), dtype=torch.float32, device="cuda")
     A.forward(d32, rig.buf_q, rig.buf_kv, out32, rig.buf_lse, rig.workspace_for(d32))
-    rig.run_forward(rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=True))
+    rig.run_forward(desc(True))
     trunc = rig.read_out_f32()
-    rig.run_forward(rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=False))
+    rig.run_forward(desc(False))
     rne = rig.read_out_f32()
     full = out32.cpu().numpy()
     assert np.array_equal(trunc, R.bf16_bits_to_f32(R.f32_to_bf16_bits_trunc(full)))
