@@ -75,7 +75,7 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
 # HBM bytes one launch of the main kernel moves (read + written), from the FETCH_SIZE and
 # WRITE_SIZE counters of rocprofv3, each scaled by what the same counter reads for the
 # calibration copy (--calib-copy-mib): fetch x2.000, write x1.000.
-MEASURED_HBM_BYTES_PER_LAUNCH = {"cfg3_global": 169.8e6 + 72.4e6}
+MEASURED_HBM_BYTES_PER_LAUNCH = {"cfg3_global": 161.1e6 + 42.5e6}
 
 
 PRODUCER_SHAPES = {   # canvas, Hq, Hkv, hd, kv_len, is_full, v_proj, ring mask: the two layer types of the 30-layer stack
