@@ -192,6 +192,42 @@ def test_split_partial_formats(gpu_ready, po, hd, hq, hkv, splits):
     assert np.array_equal(f32a[0], f32b[0])
 
 
+def test_dropped_weights_stay_below_rounding(gpu_ready, po):
+    """The kernel stores a softmax weight that is more than 2^40 below its row's running max as an exact
+    zero.  Rows built to make the most of that: one key at the top, half of the others 2^39 below it (kept),
+    half 2^41 below (dropped) and carrying values a thousand times larger than the rest.  The result still
+    meets the oracle far inside the tolerances (what is left is the bf16 rounding of the kept weights, which
+    moves ln(l) by up to 2^-8)."""
+    import torch
+    w = W.Workload("drop", 64, 8, 2, 64, 4096 - 64, rms_norm=False, seed=5)
+    q, kv = W.generate(w)
+    u = np.zeros(w.head_dim, dtype=np.float32)
+    u[:4] = 0.5                                               # |u|^2 = 1, exact in bf16
+    q[:] = u
+    ln2 = np.float32(np.log(2.0))
+    alpha = np.where(np.arange(w.t_all) % 2 == 0, (60.0 - 39.0) * ln2, (60.0 - 41.0) * ln2).astype(np.float32)
+    alpha[1000] = 60.0 * ln2
+    alpha = R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(alpha))
+    kv[0] = alpha[None, :, None] * u[None, None, :]           # score of key t = alpha[t] for every row and head
+    kv[0] = R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(kv[0])).reshape(kv[0].shape)
+    kv[1, :, 1::2, :] *= np.float32(1000.0)                   # what the dropped keys would have brought in
+    kv[1] = R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(kv[1])).reshape(kv[1].shape)
+    qd, kd = W.device_arrays(w, q, kv)
+    for splits in (1, 4):
+        desc = w.desc(n_splits=splits)
+        desc.out_dtype = capi.DG_F32
+        out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.float32, device="cuda")
+        lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+        A.forward(desc, qd, kd, out, lse, A.alloc_workspace(desc))
+        torch.cuda.synchronize()
+        od = po.make_desc(w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, layout=w.layout, t_cap=w.t_all)
+        ref, ref_lse = po.attention_f32(od, q, kv)
+        got = out.cpu().numpy().reshape(ref.shape)
+        # the dropped half would add 2048 x 2^-41 x 1000 ~ 1e-6 of a value of order one
+        assert max_abs_diff(got, ref) < 2e-3, splits              # bf16 rounding of the kept weights only
+        assert np.max(np.abs(lse.cpu().numpy().reshape(ref_lse.shape) - ref_lse)) < 4e-3, splits
+
+
 def test_scalar_and_mfma_kernels_agree_full_size(gpu_ready):
     w = W.scaled(W.config("cfg3_global"), 8192)
     q, kv = W.generate(w)
