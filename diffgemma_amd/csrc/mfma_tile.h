@@ -70,12 +70,6 @@ __device__ __forceinline__ float unpack_hi(uint32_t u) {
 // s_waitcnt as a builtin, so that the compiler's own wait-count bookkeeping sees it (gfx9
 // encoding: vmcnt = bits 3:0 and 15:14, expcnt = 6:4, lgkmcnt = 11:8; the other two counters are
 // left at their maxima).
-// wait until at most N of this wave's vector memory loads are outstanding (N <= 15)
-template <int N>
-__device__ __forceinline__ void wait_vmem_but() {
-  static_assert(N >= 0 && N <= 15, "vmcnt immediate");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
-}
 __device__ __forceinline__ void wait_vmem_all() {
   __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("" ::: "memory");
@@ -177,7 +171,7 @@ __device__ __forceinline__ TileLoad pinned(TileLoad tl) {
 
 // The loads are written as assembly on purpose: the compiler orders every LDS read after a
 // direct-to-LDS load it knows about with s_waitcnt vmcnt(0), which would expose the whole
-// fetch latency once per tile.  The kernel waits for these loads itself (wait_vmem_but).
+// fetch latency once per tile.  The kernel waits for these loads itself (wait_vmem_all).
 // All scalar operands are wave-uniform by construction; readfirstlane tells the compiler so
 // (it returns a signed int: without the casts the low half of the address would be
 // sign-extended over the high half).
