@@ -24,6 +24,9 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// NaN or infinity (a comparison with NaN is false)
+__device__ __forceinline__ bool nonfinite(float y) { return !(fabsf(y) <= 3.402823466e38f); }
+
 __device__ __forceinline__ void store_out(const AttnParams& p, size_t idx, float y) {
   if (p.out_dtype == DT_F32) {
     ((float*)p.out)[idx] = y;
@@ -90,7 +93,11 @@ __global__ void __launch_bounds__(64) attn_scalar_kernel(const AttnParams p, con
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const uint32_t d = lane + 64u * i;
-    if (d < hd) store_out(p, qoff + d, l > 0.f ? acc[i] / l : 0.f);
+    if (d < hd) {
+      const float y = l > 0.f ? acc[i] / l : 0.f;
+      if (p.dbg && nonfinite(y)) dbg_report(p.dbg, 2u, (tok << 16) | qh, d);
+      store_out(p, qoff + d, y);
+    }
   }
 }
 
@@ -160,6 +167,12 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
         }
       }
       if (!live) continue;
+      if (p.dbg) {
+        bool bad = false;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bad = bad || nonfinite(acc[e]);
+        if (bad) dbg_report(p.dbg, 2u, (tok << 16) | qh, d8 * 8u);
+      }
       if (p.out_dtype == DT_BF16) {   // eight bf16 in one 16-byte store
         const bool tr = p.out_trunc != 0;
         uint4 pk;
@@ -206,6 +219,8 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
       o.w += w * a.w;
     }
     if (!live) continue;
+    if (p.dbg && (nonfinite(o.x) || nonfinite(o.y) || nonfinite(o.z) || nonfinite(o.w)))
+      dbg_report(p.dbg, 2u, (tok << 16) | qh, d4 * 4u);
     if (p.out_dtype == DT_F32) {
       ((float4*)((float*)p.out + ooff))[d4] = o;
     } else if (p.out_dtype == DT_BF16) {   // four bf16 in one 8-byte store

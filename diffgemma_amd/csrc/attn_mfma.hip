@@ -712,6 +712,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         const float y0 = a[4 * q4] * inv, y1 = a[4 * q4 + 1] * inv;
         const float y2 = a[4 * q4 + 2] * inv, y3 = a[4 * q4 + 3] * inv;
         const size_t idx = idx0 + 8 * q4;
+        if (p.dbg && !(fabsf(y0) + fabsf(y1) + fabsf(y2) + fabsf(y3) <= 3.402823466e38f))   // NaN or infinity
+          dbg_report(p.dbg, 2u, (tok_o << 16) | qh_o, 32u * (dgrp * NDBW + i) + 4u * g2 + 8u * q4);
         if (p.out_dtype == DT_F32) {
           f32x4 v4 = {y0, y1, y2, y3};
           *(f32x4*)((float*)p.out + idx) = v4;

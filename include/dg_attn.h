@@ -150,7 +150,8 @@ typedef struct dg_debug_status {
 } dg_debug_status;
 
 #define DG_DBG_ATTN_NONPOSITIVE_L 1u  /* a row's softmax denominator was not > 0 */
-#define DG_DBG_ATTN_NONFINITE_OUT 2u  /* an output element was NaN/inf */
+#define DG_DBG_ATTN_NONFINITE_OUT 2u  /* an output element was NaN/inf (tg_id = token << 16 | query
+                                         head, value = head_dim index of the group of elements) */
 #define DG_DBG_KERNEL_ATTENTION 7u
 
 /* One layer's attention with exactly the buffers encode_layer_attention_dispatch binds:

@@ -379,6 +379,30 @@ def test_truncating_store_matches_reference_rounding(gpu_ready):
     assert np.array_equal(rne, R.bf16_bits_to_f32(R.f32_to_bf16_bits_rne(full)))
 
 
+@pytest.mark.parametrize("fixture", ["tiny", "full_grp8_hd512"])
+def test_debug_status_reports_nonfinite_output(gpu_ready, fixture):
+    """A NaN in a visible V row reaches the output; the debug status record (first writer wins) names
+    the attention kernel, a (token, head) it happened at and a head_dim index, like the reference's
+    per-step invariant check (runtime.rs:565-571).  The tiny fixture runs in one pass, the other through
+    the split path and the merge."""
+    f = FIXTURES[fixture][0]()
+    clean = A.AttnRig.from_fixture(f)
+    clean.run_dispatch(causal=0)
+    assert clean.read_debug_status().code == 0
+    kv = f.kvcache.copy()
+    hd, nkv = f.head_dim(), f.n_kv()
+    slot = f.kv_len                                          # first canvas key: visible to every row
+    kv[slot * 2 * nkv * hd + nkv * hd + 3] = np.float32(np.nan)   # V of KV head 0, element 3
+    bad = A.AttnRig.from_fixture(A.Fixture(q=f.q, kvcache=kv, layer=f.layer, canvas=f.canvas, n_q_heads=f.n_q_heads, kv_len=f.kv_len))
+    bad.run_dispatch(causal=0)
+    st = bad.read_debug_status()
+    assert (st.code, st.kernel_id) == (capi.DG_DBG_ATTN_NONFINITE_OUT, capi.DG_DBG_KERNEL_ATTENTION)
+    tok, head = st.tg_id >> 16, st.tg_id & 0xffff
+    assert tok < f.canvas and head < f.n_q_heads // nkv       # a head of the group that reads KV head 0
+    assert st.value <= 3 < st.value + 8
+    assert np.isnan(bad.read_out_f32()).any()
+
+
 def test_row_without_visible_keys(gpu_ready):
     """An empty key range stores zeros and LSE = -inf instead of NaN (attention_mma2.metal:297)."""
     import torch
