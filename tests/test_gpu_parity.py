@@ -228,6 +228,20 @@ def test_dropped_weights_stay_below_rounding(gpu_ready, po):
         assert np.max(np.abs(lse.cpu().numpy().reshape(ref_lse.shape) - ref_lse)) < 4e-3, splits
 
 
+@pytest.mark.parametrize("hd,hq,hkv", [(128, 8, 4), (512, 16, 2)])
+def test_wide_score_range_raises_reference(gpu_ready, po, hd, hq, hkv):
+    """Scores that spread over hundreds of log2 units: a row's maximum climbs by more than the 2^120 the
+    bf16 probabilities may lag behind it, so the reference is raised and the accumulators rescaled in the
+    middle of rows (with unit-variance inputs that path never runs on a bf16 cache)."""
+    w = W.Workload("wide", 64, hq, hkv, hd, 4096 - 64, rms_norm=False, q_std=12.0 * (128.0 / hd) ** 0.5, seed=17)
+    q, kv = W.generate(w)
+    s = np.einsum("d,td->t", q[0, 0], kv[0, 0]) * np.log2(np.e)          # one row's scores in log2 units
+    run_max = np.maximum.accumulate(s.reshape(-1, 32).max(axis=1))
+    assert run_max[-1] - run_max[0] > 120.0                              # the case is what it claims to be
+    for splits in (1, 0):
+        check_tolerances(*run_workload(po, w, n_splits=splits))
+
+
 def test_scalar_and_mfma_kernels_agree_full_size(gpu_ready):
     w = W.scaled(W.config("cfg3_global"), 8192)
     q, kv = W.generate(w)
