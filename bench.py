@@ -40,6 +40,9 @@ def parse_args():
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="instead of the benchmark, run the library's plain copy kernel over this many MiB "
                          "(the known-size launch the profiler's HBM byte counters are scaled by)")
+    ap.add_argument("--calib-mfma", action="store_true",
+                    help="instead of the benchmark, time the library's MFMA-only kernel with its four operand "
+                         "sets (near-constant, random, random with 75 % / 95 % of one operand zero)")
     return ap.parse_args()
 
 
@@ -496,6 +499,27 @@ def main():
         torch.cuda.synchronize()
         assert torch.equal(src, dst)
         print(json.dumps({"calib_copy_bytes": nbytes, "launches": args.steps, "kernel": "calib_copy_kernel"}))
+        return
+
+    if args.calib_mfma:
+        lib = capi.load()
+        sink = torch.zeros(256 * 256, dtype=torch.float32, device="cuda")
+        mf = C.c_uint64(0)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        names = ["near_constant", "random", "random_b_75pct_zero", "random_b_95pct_zero"]
+        rates = {}
+        for rnd in range(2):                  # every set twice, in turn: the chip warms up over the run
+            for mode, name in enumerate(names):
+                for rep in range(2):
+                    e0.record()
+                    for _ in range(8):
+                        capi.check(lib.dg_calib_mfma(sink.data_ptr(), sink.numel() * 4, 256, 8000, mode, C.byref(mf),
+                                                     A.stream_handle()))
+                    e1.record()
+                    torch.cuda.synchronize()
+                rates.setdefault(name, []).append(8 * mf.value / (e0.elapsed_time(e1) * 1e-3) / 1e12)
+        print(json.dumps({"kernel": "calib_mfma_kernel", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS,
+                          "mfma_only_tflops": rates}))
         return
 
     if args.workload in PRODUCER_SHAPES:

@@ -287,8 +287,12 @@ __global__ void calib_copy_kernel(const uint4* __restrict__ src, uint4* __restri
 typedef float calib_f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 calib_bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t calib_u32x4 __attribute__((ext_vector_type(4)));
-template <bool RANDOM>
+// MODE 0: near-constant operands; 1: random; 2 / 3: random, with 3 of 4 / 19 of 20 elements of
+// the B operand zero (what the probabilities of a long attention row look like once negligible
+// weights are dropped).
+template <int MODE>
 __global__ void __launch_bounds__(256) calib_mfma_kernel(float* sink, uint32_t iters) {
+  constexpr bool RANDOM = MODE != 0;
   calib_u32x4 a[8], b[8];
   uint32_t seed = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
   auto noise_pair = [&]() -> uint32_t {   // two bf16 of random sign, magnitude in [2^-7, 2)
@@ -306,6 +310,12 @@ __global__ void __launch_bounds__(256) calib_mfma_kernel(float* sink, uint32_t i
       // near-constant: 1 + k/128 and 1/2 - k/256 for small k (a few mantissa bits set)
       a[i][e] = RANDOM ? noise_pair() : 0x3f803f80u + ((threadIdx.x + e) & 3u);
       b[i][e] = RANDOM ? noise_pair() : 0x3f003f00u - ((threadIdx.x * 3u + e) & 3u);
+      if (MODE >= 2) {   // zero each half of the pair with probability 3/4 or 19/20
+        const uint32_t keep = MODE == 2 ? 64u : 13u;   // of 256
+        const uint32_t r = noise_pair();
+        if ((r & 255u) >= keep) b[i][e] &= 0xffff0000u;
+        if (((r >> 8) & 255u) >= keep) b[i][e] &= 0x0000ffffu;
+      }
     }
 #pragma unroll
   for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(a[i]), "+v"(b[i]));   // keep sixteen distinct fragments
@@ -331,9 +341,15 @@ __global__ void __launch_bounds__(256) calib_mfma_kernel(float* sink, uint32_t i
 
 }  // namespace
 
-hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, bool random_operands, hipStream_t s) {
-  if (random_operands) hipLaunchKernelGGL(calib_mfma_kernel<true>, dim3(workgroups), dim3(256), 0, s, sink, iters);
-  else hipLaunchKernelGGL(calib_mfma_kernel<false>, dim3(workgroups), dim3(256), 0, s, sink, iters);
+hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, uint32_t operand_mode, hipStream_t s) {
+  const dim3 grid(workgroups), block(256);
+  switch (operand_mode) {
+    case 0: hipLaunchKernelGGL(calib_mfma_kernel<0>, grid, block, 0, s, sink, iters); break;
+    case 1: hipLaunchKernelGGL(calib_mfma_kernel<1>, grid, block, 0, s, sink, iters); break;
+    case 2: hipLaunchKernelGGL(calib_mfma_kernel<2>, grid, block, 0, s, sink, iters); break;
+    case 3: hipLaunchKernelGGL(calib_mfma_kernel<3>, grid, block, 0, s, sink, iters); break;
+    default: return hipErrorInvalidValue;
+  }
   return hipGetLastError();
 }
 

@@ -124,6 +124,6 @@ hipError_t launch_topk_scores(const TopkParams& tp, uint32_t head_dim, uint32_t 
 hipError_t launch_topk_select(const TopkParams& tp, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 
 hipError_t launch_calib_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
-hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, bool random_operands, hipStream_t s);
+hipError_t launch_calib_mfma(float* sink, uint32_t workgroups, uint32_t iters, uint32_t operand_mode, hipStream_t s);
 
 }  // namespace dg

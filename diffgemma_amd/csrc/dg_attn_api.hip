@@ -590,10 +590,11 @@ int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream) {
 int dg_calib_mfma(float* sink, size_t sink_bytes, uint32_t workgroups, uint32_t iters, uint32_t random_operands,
                   uint64_t* flops, void* stream) {
   if (!sink || !flops) return DG_ERR_NULL;
+  if (random_operands > 3u) return DG_ERR_UNSUPPORTED;
   if (workgroups == 0 || iters == 0 || sink_bytes < (size_t)workgroups * 256 * sizeof(float)) return DG_ERR_WORKSPACE;
   // per workgroup: 4 waves x iters x 16 MFMAs x (32 x 32 x 16 multiply-adds)
   *flops = (uint64_t)workgroups * 4ull * iters * 16ull * (2ull * 32 * 32 * 16);
-  return dg::launch_calib_mfma(sink, workgroups, iters, random_operands != 0, (hipStream_t)stream) == hipSuccess
+  return dg::launch_calib_mfma(sink, workgroups, iters, random_operands, (hipStream_t)stream) == hipSuccess
              ? DG_OK
              : DG_ERR_LAUNCH;
 }

@@ -267,7 +267,8 @@ int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream);
  * sustains is the MFMA ceiling of the machine at hand, next to which the attention kernel's
  * rate is read.  `random_operands` = 0: near-constant operands (the multipliers draw little
  * power and the clock stays high); 1: operands of random sign, exponent and mantissa, which
- * is what attention feeds the matrix cores (the clock the chip then holds is lower).
+ * is what attention feeds the matrix cores (the clock the chip then holds is lower); 2, 3: as
+ * 1 with three quarters / 95 % of one operand's elements zero.
  * Measurement aid, no counterpart in the reference. */
 int dg_calib_mfma(float* sink, size_t sink_bytes, uint32_t workgroups, uint32_t iters, uint32_t random_operands,
                   uint64_t* flops, void* stream);
