@@ -1,4 +1,4 @@
-"""ctypes binding of include/dg_attn.h (libdg_attn_hip.so)."""
+"""ctypes binding of include/dg_attn.h and include/dg_attn_bench.h (libdg_attn_hip.so)."""
 from __future__ import annotations
 
 import ctypes as C
@@ -14,6 +14,7 @@ DG_ATTN_F_OUT_TRUNCATE = 0x1
 DG_ATTN_F_CAUSAL_SEES_MASKED = 0x2
 DG_ATTN_F_T_LO_EXPLICIT = 0x4
 DG_ATTN_F_F32_PARTIALS = 0x8
+DG_ATTN_F_F16_PARTIALS = 0x10
 DG_DBG_ATTN_NONPOSITIVE_L = 1
 DG_DBG_ATTN_NONFINITE_OUT = 2
 DG_DBG_KERNEL_ATTENTION = 7
@@ -24,7 +25,7 @@ DG_OK = 0
 DG_ERR_NULL, DG_ERR_SHAPE, DG_ERR_DTYPE, DG_ERR_LAYOUT = -1, -2, -3, -4
 DG_ERR_WORKSPACE, DG_ERR_MASK, DG_ERR_LAUNCH, DG_ERR_DEVICE, DG_ERR_UNSUPPORTED = -5, -6, -7, -8, -9
 
-# every symbol include/dg_attn.h declares
+# every symbol include/*.h declares
 EXPORTS = (
     "dg_attn_desc_reference_layout", "dg_attn_desc_head_major_layout", "dg_attn_workspace_bytes",
     "dg_attn_resolved_splits", "dg_attn_forward", "dg_attn_strerror", "dg_attn_abi_version",

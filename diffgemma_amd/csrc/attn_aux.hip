@@ -247,15 +247,31 @@ __device__ __forceinline__ float load_any(const void* src, uint32_t dt, size_t i
   if (dt == DT_BF16) return bf16_bits_to_f32(((const uint16_t*)src)[i]);
   return (float)((const _Float16*)src)[i];
 }
-__device__ __forceinline__ void store_any(void* dst, uint32_t dt, size_t i, float v) {
+// f32 -> f16 the way the reference's host wrapper rounds what it puts into the cache
+// (src/shaders/common/f16.rs:28-47): clamp to +-65504, flush subnormals to a signed zero, truncate
+// the mantissa; NaN stays NaN.
+__device__ __forceinline__ uint16_t f32_to_f16_bits_trunc(float v) {
+  const uint32_t raw = __float_as_uint(v);
+  const uint32_t sign = (raw >> 16) & 0x8000u;
+  if (v != v) return (uint16_t)(sign | 0x7E00u);
+  const uint32_t bits = __float_as_uint(fminf(fmaxf(v, -65504.f), 65504.f));
+  const int32_t new_exp = (int32_t)((bits >> 23) & 0xffu) - 127 + 15;
+  if (new_exp <= 0) return (uint16_t)sign;
+  return (uint16_t)(sign | ((uint32_t)new_exp << 10) | ((bits & 0x7fffffu) >> 13));
+}
+// f32 sources are rounded like the reference's wrapper around its CPU attention does
+// (src/shaders/attn/attention/mod.rs:218-240): bf16 and f16 by truncation.  16-bit sources are
+// copied exactly when the types match and widened/narrowed by the hardware conversion otherwise.
+__device__ __forceinline__ void store_any(void* dst, uint32_t dt, size_t i, float v, bool from_f32) {
   if (dt == DT_F32) ((float*)dst)[i] = v;
-  else if (dt == DT_BF16) ((uint16_t*)dst)[i] = f32_to_bf16_bits(v, false);
+  else if (dt == DT_BF16) ((uint16_t*)dst)[i] = f32_to_bf16_bits(v, from_f32);
+  else if (from_f32) ((uint16_t*)dst)[i] = f32_to_f16_bits_trunc(v);
   else ((_Float16*)dst)[i] = (_Float16)v;
 }
 
 __global__ void convert_kernel(const void* src, uint32_t sdt, void* dst, uint32_t ddt, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-    store_any(dst, ddt, i, load_any(src, sdt, i));
+    store_any(dst, ddt, i, load_any(src, sdt, i), sdt == DT_F32);
 }
 
 __global__ void kv_gather_kernel(const void* src, uint32_t sdt, void* dst, uint32_t ddt, uint32_t hkv,
@@ -267,7 +283,7 @@ __global__ void kv_gather_kernel(const void* src, uint32_t sdt, void* dst, uint3
     const uint32_t t = (uint32_t)((i / hd) % t_all);
     const uint32_t h = (uint32_t)(i / ((size_t)hd * t_all));
     const int64_t s = (int64_t)kv_slot(ring_mask, t) * tok_stride + (int64_t)h * head_stride + d;
-    store_any(dst, ddt, i, load_any(src, sdt, (size_t)s));
+    store_any(dst, ddt, i, load_any(src, sdt, (size_t)s), sdt == DT_F32);
   }
 }
 

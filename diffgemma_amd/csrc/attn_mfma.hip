@@ -34,9 +34,10 @@
 // together with P.  Rescaling O costs about as much as the tile's P.V MFMAs, and with unit-RMS
 // Q and K and no 1/sqrt(d) the scores of a row spread over tens of log2 units, so a small tau
 // would rescale some row block on almost every tile.  Any reference below the true max is
-// exact as long as nothing overflows: P <= 2^tau, and the fp32 sums stay below
-// 2^tau * keys * |v|, far from 2^127 for tau = 80.  With f16 operands P itself has to stay
-// below 65504: tau = 15.
+// exact as long as nothing overflows.  bf16: tau = 120 with the probabilities stored as
+// 2^(score - reference - 86), so P <= 2^34 and the fp32 sums stay below 2^34 * keys * |v|, far
+// from 2^127; a weight more than 2^40 below the row's running max is stored as an exact zero.
+// With f16 operands P itself has to stay below 65504: tau = 15, no offset.
 #include "attn_params.h"
 #include "mfma_tile.h"
 
@@ -60,26 +61,6 @@ constexpr float kTau = F16 ? 15.0f : 120.0f;
 template <bool F16>
 constexpr float kPOff = F16 ? 0.0f : 86.0f;
 constexpr float kDrop = 40.0f;
-
-// Optional per-phase cycle accounting (development builds only): every wave sums the cycles
-// it spends in each phase of the tile loop and stores the sums at the end.
-#ifdef DG_ATTN_PHASE_TIMING
-#define DG_PHASE_DECL unsigned long long ph_t = clock64(), ph_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#define DG_PHASE(i)                          \
-  {                                          \
-    const unsigned long long now = clock64(); \
-    ph_acc[i] += now - ph_t;                 \
-    ph_t = now;                              \
-  }
-#define DG_PHASE_STORE                                                                    \
-  if (p.phase_cycles && lane == 0) {                                                      \
-    for (int i = 0; i < 8; ++i) p.phase_cycles[((size_t)blockIdx.x * 4 + wave) * 8 + i] = ph_acc[i]; \
-  }
-#else
-#define DG_PHASE_DECL
-#define DG_PHASE(i)
-#define DG_PHASE_STORE
-#endif
 
 // Score MFMAs, written as assembly so that their accumulator is an ordinary VGPR tuple.  O fills
 // all 256 accumulation registers at head_dim 512; the compiler gives every MFMA of such a
@@ -123,12 +104,6 @@ __device__ __forceinline__ void scale_acc4(float& x0, float& x1, float& x2, floa
       : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
       : "v"(c));
 }
-#ifdef DG_ATTN_PHASE_TIMING
-__device__ __forceinline__ float touch_acc(float x) {
-  asm volatile("s_nop 0" : "+a"(x));
-  return x;
-}
-#endif
 // dst = src for a score tile, as instructions the compiler cannot move or merge away; part I of
 // 8 copies elements 2 I and 2 I + 1
 template <int I>
@@ -150,6 +125,9 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v) {
   asm volatile("" : "+v"(v));
   return v;
 }
+
+// the value brought into the finite range of f16 (NaN stays NaN)
+__device__ __forceinline__ float sat_f16(float x) { return __builtin_amdgcn_fmed3f(x, -65504.f, 65504.f); }
 
 // acc + lo + hi of a packed pair, in one dot-product instruction
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -335,7 +313,6 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
 
-  DG_PHASE_DECL
   if (ntile > 0) {
     lds_char* const k0 = (lds_char*)(smem + OFF_K0);
     lds_char* const k1 = (lds_char*)(smem + OFF_K1);
@@ -494,7 +471,6 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     __syncthreads();   // every wave is done with K(tb): its buffer takes K(tb+2)
     issue_tile<D, false>(k_load((tb + 2) * kBlockN, k0, lane), wave, lane);
     kf_preload(k1);
-    DG_PHASE(0)
 
     for (uint32_t jj = 0; jj < ntile; ++jj) {
       const uint32_t par = jj & 1u;
@@ -511,7 +487,6 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       if constexpr (NSPLIT == 0)
         static_for<0, NCH>([&](auto c_c) { softmax_piece(c_c, s_a, t0, par); });
       qk_steps(I0{}, ISPLIT{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par, nothing);
-      DG_PHASE(3)
       // The one barrier of the tile.  Before it: this wave's loads of V(jj) and K(jj+2), issued
       // during the previous tile's P.V, have landed, its P is written and the last K fragments
       // of the tile are in registers (the barrier's fence waits for all three).  After it: P,
@@ -519,9 +494,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // reading K(jj+1), V(jj-1) and the previous tile's P (which has its own buffer), so their
       // buffers can be refilled.
       wait_vmem_all();
-      DG_PHASE(4)
       __syncthreads();
-      DG_PHASE(5)
 
       // ---- d-owner role ----
       lds_char* const pbuf = (lds_char*)(smem + OFF_P) + par * P_BYTES;
@@ -586,9 +559,6 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // the softmax expects them; behind the last MFMAs, the reads of the first K fragments of
       // tile jj+2 (pinned there: at the loop end the compiler would move them to the top of the
       // next iteration, in front of the MFMAs that wait for them).
-#ifdef DG_FINE_PHASES
-      DG_PHASE(1)
-#endif
       constexpr int COPY_AT = NPV >= 16 ? NPV / 2 : 0;   // MFMA index after which the copy starts
       static_for<0, NVF>([&](auto f_c) {
         constexpr int f = decltype(f_c)::value, ks = f / NDBW, i = f % NDBW;
@@ -610,17 +580,12 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (NPV < 16) static_for<0, 8>([&](auto i_c) { copy_scores_part<decltype(i_c)::value>(s_a, s_b); });
       if constexpr (NPV < PFK) kf_preload(kb_next2);
-#ifdef DG_ATTN_PHASE_TIMING
-      o[0][0] = touch_acc(o[0][0]);   // the accumulators have to exist before the clock is read
-#endif
-      DG_PHASE(6)
     }
     // the loads issued for tiles after the last one must not outlive this workgroup's LDS
     wait_vmem_all();
   }
 
   // ---- epilogue ----
-  DG_PHASE_STORE
   // row owners publish (m, l) of their rows; d owners normalise and store their slice of O
   const float l_tot = sum_across_halves(l_part + l_part2);
   const float m_pub = m_ref + kPOff<F16>;   // the exponent the sums are relative to
@@ -657,8 +622,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
           u32x2 h2;
-          h2[0] = pack2<true>(a[4 * q4] * inv, a[4 * q4 + 1] * inv);
-          h2[1] = pack2<true>(a[4 * q4 + 2] * inv, a[4 * q4 + 3] * inv);
+          h2[0] = pack2<true>(sat_f16(a[4 * q4] * inv), sat_f16(a[4 * q4 + 1] * inv));
+          h2[1] = pack2<true>(sat_f16(a[4 * q4 + 2] * inv), sat_f16(a[4 * q4 + 3] * inv));
           *(__attribute__((address_space(3))) u32x2*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 2) = h2;
         }
       }

@@ -26,7 +26,6 @@ struct AttnParams {
                        // index space in f16 holding accumulators divided by the split's row sum
   float* part_ml;      // [split][hkv][rows_pad][2] (m in log2 units, l)
   uint32_t* dbg;       // 4 words, first-writer-wins, or null
-  unsigned long long* phase_cycles;  // [workgroup][wave][8] cycle sums; only written by builds with DG_ATTN_PHASE_TIMING
   int64_t k_tok_stride, k_head_stride, v_tok_stride, v_head_stride;  // elements
   uint32_t canvas, hq, hkv, group;
   uint32_t kv_len, t_all;

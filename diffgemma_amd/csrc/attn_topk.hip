@@ -26,29 +26,6 @@ namespace {
 
 constexpr int kCandCap = 2048;     // LDS candidate list of the select kernel (sized for 4 workgroups per CU)
 
-// Optional per-phase cycle accounting of the select kernel (development builds only): thread 0 of
-// every workgroup adds the cycles it spent in each phase to eight global sums.
-#ifdef DG_ATTN_PHASE_TIMING
-#define TK_PHASE_DECL unsigned long long tk_t = clock64();
-#define TK_PHASE(i)                                                        \
-  if (p.phase_cycles && tid == 0) {                                        \
-    const unsigned long long now = clock64();                              \
-    atomicAdd(&p.phase_cycles[i], now - tk_t);                             \
-    tk_t = now;                                                            \
-  }
-#define SC_PHASE(i)                                                        \
-  if (p.phase_cycles && threadIdx.x == 0) {                                \
-    const unsigned long long now = clock64();                              \
-    atomicAdd(&p.phase_cycles[8 + (i)], now - sc_t);                       \
-    sc_t = now;                                                            \
-  }
-#define SC_PHASE_DECL unsigned long long sc_t = clock64();
-#else
-#define TK_PHASE_DECL
-#define TK_PHASE(i)
-#define SC_PHASE(i)
-#define SC_PHASE_DECL
-#endif
 // radix digits of the 32-bit key, most significant first: 11 + 11 + 10 bits
 __device__ __forceinline__ uint32_t digit_shift(int level) { return level == 0 ? 21u : level == 1 ? 10u : 0u; }
 __device__ __forceinline__ uint32_t digit_bits(int level) { return level == 2 ? 10u : 11u; }
@@ -174,8 +151,6 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
     row_off[e] = ((hh * tp.ntok + tl) * tp.t_pad + l32) * 4u;
     row_mask |= ok ? 1u << e : 0u;
   }
-
-  SC_PHASE_DECL
 #pragma unroll
   for (int i = 0; i < PF; ++i) issue_k(tb + i);
   // lane l32 holds key t0 + l32 of sixteen rows; element e of a tile's scores goes to
@@ -198,9 +173,7 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
     // first half of this tile's MFMAs: stores count in the same counter as the loads, and issued
     // right before the wait they would have to drain first; issued here they are at least half
     // a tile old at the next wait, and their address arithmetic hides behind the matrix pipe.
-    SC_PHASE(0)
     wait_loads_then_barrier<(PF - 1) * NLD>();
-    SC_PHASE(1)
     const bool have_prev = j > tb;
     // (the loads of K(j+PF) are issued between the MFMAs below: back to back each of them holds
     // the wave's issue slot for about two MFMAs' worth of cycles)
@@ -253,10 +226,8 @@ __global__ void __launch_bounds__(256) topk_scores_kernel(const TopkParams tp) {
       __builtin_amdgcn_sched_barrier(0);
     });
     s_prev = s;
-    SC_PHASE(2)
   }
   store_tile(s_prev, te - 1u);
-  SC_PHASE(3)
   wait_vmem_all();   // no direct-to-LDS load may outlive the workgroup's LDS
 }
 
@@ -429,8 +400,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
       }
     }
   };
-
-  TK_PHASE_DECL
   if (tid == 0) {
     sh.n_sel = 0;
     sh.n_cand = 0;
@@ -469,10 +438,8 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
       const uint64_t want = min<uint64_t>(5ull * k / 2ull, 3ull * kCandCap / 4ull);
       const uint32_t r = min(m, (uint32_t)((want * m + n_valid - 1ull) / n_valid) + 8u);
       uint32_t te, ne;
-      TK_PHASE(7)
       const uint32_t tau = lds_kth_largest(
           sh, m, r, tid, [&](uint32_t i, uint32_t& key) { key = sh.cand_key[i]; return true; }, &te, &ne);
-      TK_PHASE(1)
       scan_row([&](uint32_t t, float sv) {
         const uint32_t key = score_key(sv);
         if (key >= tau) {
@@ -511,8 +478,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
     class_count = sh.res[2];
     __syncthreads();
   }
-
-  TK_PHASE(0)
   if (class_count > (uint32_t)kCandCap) {
     // More than a list's worth of bit-identical scores at the threshold (a degenerate row, e.g.
     // an all-zero query).  Keys above go in as they come; of the ties the first `remaining` by
@@ -570,7 +535,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
       });
       __syncthreads();
     }
-    TK_PHASE(1)
     const uint32_t n_cand = min(sh.n_cand, (uint32_t)kCandCap);
 
     // ---- the k-th key among the candidates: the levels not yet done, over the list ----
@@ -600,7 +564,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
       n_eq = cls;
     }
     // thr is the k-th largest key; take_eq of the n_eq keys equal to it are kept
-    TK_PHASE(6)
 
     // ---- equal scores: the lower positions win.  Threshold on position by the same select ----
     uint32_t t_key_min = 0u;   // ties with ~t >= t_key_min are kept
@@ -627,8 +590,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
     }
     __syncthreads();
   }
-
-  TK_PHASE(2)
   // ---- sort the kept keys by position (bitonic, padded with +inf positions) ----
   uint32_t npow = 1;
   while (npow < k) npow <<= 1;
@@ -655,8 +616,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
       __syncthreads();
     }
   }
-
-  TK_PHASE(3)
   // ---- softmax over the kept scores (cpu.rs:95-104) ----
   float* const fred = (float*)sh.hist;   // histogram storage is free now
   float m = -INFINITY;
@@ -683,8 +642,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
   }
   const float lsum = fred[0];
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
-
-  TK_PHASE(4)
   // ---- gathered P.V: wave w takes kept keys w, w+4, ...; a lane owns PER consecutive d ----
   constexpr int PER = D >= 64 ? D / 64 : 1;
   const bool lane_on = lane * PER < (uint32_t)D;
@@ -741,7 +698,6 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
       }
     }
   }
-  TK_PHASE(5)
   if (lane_on) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) red[wave][lane * PER + i] = acc[i];

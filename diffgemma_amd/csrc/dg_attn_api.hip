@@ -1,6 +1,7 @@
 // extern "C" boundary of libdg_attn_hip.so: descriptor validation, launch planning, and the
 // reference-shaped dispatch entry.  No allocation, no host synchronisation, no exceptions.
 #include "../../include/dg_attn.h"
+#include "../../include/dg_attn_bench.h"
 
 #include <hip/hip_runtime.h>
 
@@ -28,10 +29,6 @@ DeviceInfo g_dev[64];
 thread_local uint32_t* g_tls_dbg = nullptr;
 std::mutex g_dev_mu;
 
-#ifdef DG_ATTN_PHASE_TIMING
-unsigned long long* g_phase_cycles = nullptr;
-#endif
-
 struct ProfState {
   std::vector<hipEvent_t> ev;
   uint32_t used = 0;
@@ -53,6 +50,14 @@ int device_info(DeviceInfo* out) {
   if (di.checked < 0) return DG_ERR_DEVICE;
   *out = di;
   return DG_OK;
+}
+
+// Compute units the launch plans are made for: those of the current device when it is a
+// gfx950 part, else (no device: host-side sizing and tests) the 256 of an MI355X.  Sizing calls
+// and launches use the same number, so a workspace sized by the library always fits its launch.
+int plan_cus() {
+  DeviceInfo di;
+  return device_info(&di) == DG_OK ? di.cus : 256;
 }
 
 // Everything the launch needs that can be derived on the host without a device.
@@ -95,7 +100,10 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
   pl->e_dtype = d->kv_dtype == DG_BF16 ? DG_BF16 : DG_F16;
   pl->gather_kv = d->kv_dtype == DG_F32;
   if (d->q_dtype == DG_F32) {
+    // f32 queries become bf16 by truncation, the reference wrapper's rounding of Q
+    // (src/shaders/attn/attention/mod.rs:218-240), whatever the cache holds
     pl->convert_q = true;
+    pl->q_is_bf16 = pl->e_dtype == DG_F16;
   } else if (d->q_dtype == DG_BF16 && pl->e_dtype == DG_F16) {
     pl->q_is_bf16 = true;  // bf16 activations over an f16 cache: the reference's own pairing
   } else if (d->q_dtype != pl->e_dtype) {
@@ -219,8 +227,7 @@ void dg_attn_desc_head_major_layout(dg_attn_desc* d, uint64_t t_cap) {
 int dg_attn_workspace_bytes(const dg_attn_desc* d, size_t* out_bytes) {
   if (!d || !out_bytes) return DG_ERR_NULL;
   Plan pl;
-  // Sized for a 256-CU part whatever device is current, so the answer does not depend on it.
-  const int rc = make_plan(d, 256, &pl);
+  const int rc = make_plan(d, plan_cus(), &pl);
   if (rc != DG_OK) return rc;
   *out_bytes = pl.total;
   return DG_OK;
@@ -229,7 +236,7 @@ int dg_attn_workspace_bytes(const dg_attn_desc* d, size_t* out_bytes) {
 int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits) {
   if (!d || !out_splits) return DG_ERR_NULL;
   Plan pl;
-  const int rc = make_plan(d, 256, &pl);
+  const int rc = make_plan(d, plan_cus(), &pl);
   if (rc != DG_OK) return rc;
   *out_splits = pl.n_splits;
   return DG_OK;
@@ -238,7 +245,7 @@ int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits) {
 int dg_attn_visible_pairs(const dg_attn_desc* d, uint64_t* pairs, double* flops) {
   if (!d) return DG_ERR_NULL;
   Plan pl;
-  const int rc = make_plan(d, 256, &pl);
+  const int rc = make_plan(d, plan_cus(), &pl);
   if (rc != DG_OK) return rc;
   uint64_t n = 0;
   for (uint32_t tok = 0; tok < d->canvas; ++tok) {
@@ -276,7 +283,7 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   p.q = q;
   p.ring_mask = d->kv_ring_mask;
   if (pl.convert_q) {
-    if (dg::launch_convert(q, d->q_dtype, ws + pl.off_q, pl.e_dtype, (size_t)d->canvas * d->n_q_heads * hd, s) != hipSuccess)
+    if (dg::launch_convert(q, d->q_dtype, ws + pl.off_q, DG_BF16, (size_t)d->canvas * d->n_q_heads * hd, s) != hipSuccess)
       return DG_ERR_LAUNCH;
     p.q = ws + pl.off_q;
   }
@@ -325,7 +332,9 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   p.q_is_bf16 = pl.q_is_bf16 ? 1u : 0u;
   p.out_dtype = d->out_dtype;
   p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
-  p.part_half = (pl.n_splits > 1 && d->out_dtype != DG_F32 && !(d->flags & DG_ATTN_F_F32_PARTIALS))
+  // f16 partial rows need |V| <= 65504: an f16 cache guarantees it, for a bf16 cache the caller says so
+  p.part_half = (pl.n_splits > 1 && d->out_dtype != DG_F32 && !(d->flags & DG_ATTN_F_F32_PARTIALS) &&
+                 (pl.e_dtype == DG_F16 || (d->flags & DG_ATTN_F_F16_PARTIALS)))
                     ? 1u
                     : 0u;
   p.scale_log2 = pl.scale * dg::kLog2e;
@@ -341,7 +350,7 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
   int rc = device_info(&di);
   if (rc != DG_OK) return rc;
   Plan pl;
-  rc = make_plan(d, 256, &pl);
+  rc = make_plan(d, di.cus, &pl);
   if (rc != DG_OK) return rc;
   if (pl.total > 0 && (!workspace || workspace_bytes < pl.total)) return DG_ERR_WORKSPACE;
   if (pl.total > 0 && ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
@@ -358,9 +367,6 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
     p.part_ml = (float*)(ws + pl.off_part_ml);
   }
   p.dbg = g_tls_dbg;  // set only while dg_attention_dispatch is on the stack
-#ifdef DG_ATTN_PHASE_TIMING
-  p.phase_cycles = g_phase_cycles;
-#endif
 
   if (pl.scalar) {
     if (dg::launch_attn_scalar(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
@@ -413,7 +419,7 @@ int make_topk_plan(const dg_attn_desc* d, const uint32_t* k_cfg, const Plan& pl,
 int dg_attn_topk_workspace_bytes(const dg_attn_desc* d, const uint32_t* k_cfg, size_t* out_bytes) {
   if (!d || !out_bytes) return DG_ERR_NULL;
   Plan pl;
-  int rc = make_plan(d, 256, &pl);
+  int rc = make_plan(d, plan_cus(), &pl);
   if (rc != DG_OK) return rc;
   TopkPlan tk;
   rc = make_topk_plan(d, k_cfg, pl, &tk);
@@ -429,7 +435,7 @@ int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const voi
   int rc = device_info(&di);
   if (rc != DG_OK) return rc;
   Plan pl;
-  rc = make_plan(d, 256, &pl);
+  rc = make_plan(d, plan_cus(), &pl);
   if (rc != DG_OK) return rc;
   TopkPlan tk;
   rc = make_topk_plan(d, k_cfg, pl, &tk);
@@ -443,9 +449,6 @@ int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const voi
   rc = fill_params(d, pl, q, kv_base, out, nullptr, nullptr, s, &tp.a);   // no conversion passes: dtypes checked above
   if (rc != DG_OK) return rc;
   tp.a.dbg = g_tls_dbg;
-#ifdef DG_ATTN_PHASE_TIMING
-  tp.a.phase_cycles = g_phase_cycles;
-#endif
   tp.s_plane = (float*)workspace;
   tp.t_pad = tk.t_pad;
   tp.tile_first = pl.tile_first;
@@ -460,7 +463,7 @@ int dg_attn_topk_forward(const dg_attn_desc* d, const uint32_t* k_cfg, const voi
     // enough workgroups for every CU, no split shorter than 8 key tiles; splits write disjoint
     // columns of the score plane, so there is nothing to merge
     const uint32_t base = d->n_kv_heads * tp.n_mtiles;
-    uint32_t splits = std::max(1u, (256u + base - 1u) / base);
+    uint32_t splits = std::max(1u, ((uint32_t)di.cus + base - 1u) / base);
     tp.n_splits = std::max(1u, std::min(splits, ntiles / 8u));
     // (timing aid: one event pair per kernel, scores first)
     const bool prof = g_prof.active && 2 * (size_t)g_prof.used + 3 < g_prof.ev.size();
@@ -537,11 +540,6 @@ int dg_attention_topk_dispatch(const void* q, const void* kvcache, void* out, co
   g_tls_dbg = nullptr;
   return rc;
 }
-
-#ifdef DG_ATTN_PHASE_TIMING
-// development builds only: device buffer of [workgroups][4][8] cycle sums
-void dg_debug_set_phase_buffer(void* device_ptr) { g_phase_cycles = (unsigned long long*)device_ptr; }
-#endif
 
 int dg_prof_begin(uint32_t max_launches) {
   if (g_prof.active) return DG_ERR_UNSUPPORTED;

@@ -143,8 +143,10 @@ __device__ __forceinline__ TileLoad make_tile_load(const char* head_base, int64_
   TileLoad tl;
   tl.base = head_base + (int64_t)kv_slot(ring_mask, t0) * tok_stride_b;
   tl.stride_b = (uint32_t)tok_stride_b;
-  tl.rmin = FIRST && t_min > t0 ? t_min - t0 : 0u;
   tl.rmax = min(t_all - 1u - t0, (uint32_t)kBlockN - 1u);
+  // (a first visible key at or past t_all, i.e. rows that see nothing, must not move the clamp
+  // past the last key that exists)
+  tl.rmin = FIRST && t_min > t0 ? min(t_min - t0, tl.rmax) : 0u;
   tl.lds = (uint32_t)(size_t)buf;
   if constexpr (L::PAD) {
     tl.lds += wave * (IS_V ? L::V_STRIDE : L::K_STRIDE);

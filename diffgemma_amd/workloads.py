@@ -54,6 +54,10 @@ class Workload:
             t_lo = self.t_lo
         if self.sees_masked:
             flags |= capi.DG_ATTN_F_CAUSAL_SEES_MASKED
+        if not flags & capi.DG_ATTN_F_F32_PARTIALS:
+            # every generator below draws V from N(0, kv_std^2) (RMS-normalised or not): far inside the
+            # f16 range, as are the V rows a model's cache holds after the producer's RMSNorm
+            flags |= capi.DG_ATTN_F_F16_PARTIALS
         args = dict(causal_rows=self.causal_rows, window=self.window, q_dtype=dt,
                     kv_dtype=capi.DG_F16 if self.kv_f16 else dt,
                     out_dtype=dt, flags=flags, t_lo=t_lo, layout=self.layout, t_cap=self.t_all)

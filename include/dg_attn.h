@@ -61,13 +61,18 @@ typedef enum dg_kernel_sel {
 #define DG_ATTN_F_CAUSAL_SEES_MASKED 0x2u  /* causal rows also see canvas keys >= kv_len+causal_rows */
 #define DG_ATTN_F_T_LO_EXPLICIT 0x4u       /* non-causal rows start at desc.t_lo instead of the
                                               window rule kv_len-(window-1) */
-#define DG_ATTN_F_F32_PARTIALS 0x8u        /* keep split partial rows in fp32.  Default with a 16-bit
-                                              output: partial rows travel between the attention and
-                                              the merge kernel as f16 after division by the split's
-                                              row sum (a weighted mean of V rows, so it needs
-                                              |V| <= 65504, which an f16 cache guarantees; the
-                                              rounding is 1/8 of the output's).  f32 outputs always
-                                              use fp32 partials. */
+#define DG_ATTN_F_F32_PARTIALS 0x8u        /* keep split partial rows in fp32 (always the case with an
+                                              f32 output) */
+#define DG_ATTN_F_F16_PARTIALS 0x10u       /* bf16 cache, 16-bit output: let split partial rows travel
+                                              between the attention and the merge kernel as f16 after
+                                              division by the split's row sum (a weighted mean of V
+                                              rows).  The caller asserts |V| <= 65504 and accepts that
+                                              partial-row values below 2^-14 lose precision; true of
+                                              every cache the producer below writes (V rows are
+                                              RMS-normalised, |v| <= sqrt(head_dim)).  Values beyond
+                                              the range saturate.  This is the default for an f16
+                                              cache, which guarantees the range; the rounding is 1/8 of
+                                              a bf16 output's. */
 
 typedef struct dg_attn_desc {
   uint32_t canvas;        /* query rows; the reference passes active_canvas (256/128/64) */
@@ -108,7 +113,10 @@ int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits);
 
 /* q, out: [canvas][n_q_heads][head_dim]; lse: [canvas][n_q_heads] fp32 natural-log
  * log-sum-exp of the scaled scores (NULL to skip; a row with no visible key gets -inf and
- * an all-zero output row). */
+ * an all-zero output row).  Accuracy of lse: the row sum is taken over the probabilities as
+ * rounded to the MFMA operand type (the numbers P.V multiplies, so that out is an exact
+ * weighted mean), which moves ln(sum) by at most 2^-8 absolute: |lse - exact| <=
+ * max(1e-3 |exact|, 2^-8). */
 int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
                     void* workspace, size_t workspace_bytes, void* stream);
 
@@ -241,37 +249,6 @@ int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void*
 
 #define DG_DBG_ROPE_NONFINITE 3u        /* a head's 1/rms was not finite */
 #define DG_DBG_KERNEL_QK_ROPE_KV 6u
-
-/* ---- optional kernel timing (measurement aid; no counterpart in the reference, whose
- * harness times whole command buffers: src/shaders/attn/harness.rs:149-170) ----
- * Between dg_prof_begin and dg_prof_end every dg_attn_forward issued by the calling thread
- * records one HIP event pair on its stream around the main attention kernel only (the
- * merge and conversion kernels stay outside the pair).  dg_prof_end waits for the last
- * recorded event, returns the summed kernel time and releases the events. */
-int dg_prof_begin(uint32_t max_launches);
-int dg_prof_end(double* main_kernel_ms_total, uint32_t* n_launches);
-/* dg_attn_topk_forward records two pairs per block of canvas rows instead: one around the score
- * kernel, then one around the select kernel.  dg_prof_end_split ends the session like dg_prof_end
- * and returns the time of the even-numbered pairs (0, 2, ...: the score kernels of a top-k
- * session) and of the odd-numbered ones (the select kernels) separately. */
-int dg_prof_end_split(double* even_ms_total, double* odd_ms_total, uint32_t* n_pairs);
-
-/* Plain device-to-device copy of `bytes` (multiple of 16) with a kernel of this library: a
- * launch of known HBM traffic (bytes read + bytes written) that the FETCH_SIZE / WRITE_SIZE
- * profiler counters are scaled by.  Measurement aid, no counterpart in the reference. */
-int dg_calib_copy(void* dst, const void* src, size_t bytes, void* stream);
-
-/* Launch of nothing but bf16 32x32x16 MFMAs (`workgroups` x 4 waves x `iters` x 16) writing
- * `*flops` = the floating-point operations it performs; the caller times it.  `sink` (at
- * least workgroups*256 floats, device memory) is never written in practice.  What this
- * sustains is the MFMA ceiling of the machine at hand, next to which the attention kernel's
- * rate is read.  `random_operands` = 0: near-constant operands (the multipliers draw little
- * power and the clock stays high); 1: operands of random sign, exponent and mantissa, which
- * is what attention feeds the matrix cores (the clock the chip then holds is lower); 2, 3: as
- * 1 with three quarters / 95 % of one operand's elements zero.
- * Measurement aid, no counterpart in the reference. */
-int dg_calib_mfma(float* sink, size_t sink_bytes, uint32_t workgroups, uint32_t iters, uint32_t random_operands,
-                  uint64_t* flops, void* stream);
 
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);

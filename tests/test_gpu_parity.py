@@ -69,6 +69,55 @@ def test_reference_fixture_unrounded_and_lse(gpu_ready, po, name):
     assert np.max(np.abs(lse - want_lse) / np.maximum(np.abs(want_lse), 1.0)) < LSE_REL
 
 
+@pytest.mark.parametrize("name", ["tiny", "wide", "sliding_hd256"])
+def test_f32_inputs_are_rounded_like_the_reference_wrapper(gpu_ready, po, name):
+    """f32 queries and an f32 cache handed to dg_attn_forward are brought down on the device the way the
+    reference's wrapper rounds them on the host (attention/mod.rs:218-240: Q -> bf16, K/V -> f16, both by
+    truncation, f16 with clamp and subnormal flush): the result equals, bit for bit, the call fed the
+    host-rounded bits, and meets the wrapper's own oracle."""
+    import torch
+    f = FIXTURES[name][0]()
+    _, want, _ = reference_cpu(po, f)
+    rig = A.AttnRig.from_fixture(f, kv_slack_slots=0)            # host-rounded bf16 Q / f16 cache
+    d16 = rig.desc(kernel=capi.DG_KERNEL_MFMA, truncate=False)
+    d16.out_dtype = capi.DG_F32
+    out16 = torch.zeros(f.out_len(), dtype=torch.float32, device="cuda")
+    A.forward(d16, rig.buf_q, rig.buf_kv, out16, rig.buf_lse, rig.workspace_for(d16))
+    # the same fixture as f32, with values the f16 conversion has to clamp, flush and truncate
+    q32 = torch.from_numpy(np.ascontiguousarray(f.q, dtype=np.float32)).cuda()
+    kv32 = torch.from_numpy(np.ascontiguousarray(f.kvcache, dtype=np.float32)).cuda()
+    d32 = A.make_desc(f.canvas, f.n_q_heads, f.n_kv(), f.head_dim(), f.kv_len, q_dtype=capi.DG_F32,
+                      kv_dtype=capi.DG_F32, out_dtype=capi.DG_F32, kernel=capi.DG_KERNEL_MFMA,
+                      kv_region_bytes=2 * f.layer.kv_region)   # the region offset is in bytes: f32 elements are twice as wide
+    out32 = torch.zeros(f.out_len(), dtype=torch.float32, device="cuda")
+    lse32 = torch.zeros(f.canvas * f.n_q_heads, dtype=torch.float32, device="cuda")
+    A.forward(d32, q32, kv32, out32, lse32, A.alloc_workspace(d32))
+    torch.cuda.synchronize()
+    assert torch.equal(out16, out32)
+    assert max_abs_diff(out32.cpu().numpy(), want) < 2e-4
+
+
+def test_f32_cache_conversion_clamps_flushes_and_truncates(gpu_ready, po):
+    """Values the three rules of the reference's f16 conversion act on (src/shaders/common/f16.rs:28-47):
+    beyond +-65504 (clamped, not infinity), below 2^-14 (flushed to a signed zero), and mantissas that
+    round-to-nearest would round up (truncated).  V carries them; the output of a one-key row is that V row."""
+    import torch
+    hd = 32
+    v = np.zeros(hd, dtype=np.float32)
+    v[:8] = [1e6, -1e6, 3e-5, -3e-5, 1.0 + 2.0 ** -11 + 2.0 ** -12, -(2.0 + 2.0 ** -10 + 2.0 ** -11), 65504.0, 7e-8]
+    want = R.f16_bits_to_f32(R.f32_to_f16_bits_trunc(v))
+    assert want[0] == 65504.0 and want[2] == 0.0 and want[4] == 1.0     # the rules do act on these values
+    kv = np.zeros((1, 2, 1, hd), dtype=np.float32)               # one slot: [K head | V head]
+    kv[0, 0, 0, 0] = 1.0
+    kv[0, 1, 0] = v
+    q = np.ones((1, 1, hd), dtype=np.float32)
+    d = A.make_desc(1, 1, 1, hd, 0, q_dtype=capi.DG_F32, kv_dtype=capi.DG_F32, out_dtype=capi.DG_F32)
+    out = torch.zeros(hd, dtype=torch.float32, device="cuda")
+    A.forward(d, torch.from_numpy(q.ravel()).cuda(), torch.from_numpy(kv.ravel()).cuda(), out, None, A.alloc_workspace(d))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
 def test_model_full_fixture_midsize(gpu_ready, po):
     """The reference's bench fixture (attention_gemm/mod.rs:364-432) at a prefix that spans many key tiles."""
     f = A.model_full_fixture(1000, canvas=64)
@@ -174,8 +223,9 @@ def test_split_count_invariance_full_size(gpu_ready):
 @pytest.mark.parametrize("hd,hq,hkv,splits", [(32, 8, 4, 17), (64, 32, 4, 9), (128, 8, 4, 33), (256, 16, 8, 8), (256, 16, 8, 64),
                                               (512, 16, 2, 8), (512, 8, 1, 40)])
 def test_split_partial_formats(gpu_ready, po, hd, hq, hkv, splits):
-    """Split partial rows travel as normalised f16 rows by default with a 16-bit output
-    (DG_ATTN_F_F32_PARTIALS keeps fp32): both formats meet the oracle, they differ by output roundings
+    """Split partial rows travel as normalised f16 rows with a 16-bit output when the cache is f16 or the
+    caller vouches for the range of a bf16 one (DG_ATTN_F_F16_PARTIALS, which the workload descriptors set;
+    DG_ATTN_F_F32_PARTIALS keeps fp32): both formats meet the oracle, they differ by output roundings
     only, and an f32 output keeps fp32 partials.  The split counts are larger than head_dim / 8 and
     head_dim / 4: the merge reads every split's weight whatever lanes its loads keep busy."""
     w = W.Workload("partials", 100, hq, hkv, hd, 2049, causal_rows=50, seed=11)

@@ -15,7 +15,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def header_functions():
-    text = open(os.path.join(ROOT, "include", "dg_attn.h")).read()
+    inc = os.path.join(ROOT, "include")
+    text = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(dg_[a-z0-9_]+)\s*\(", text)))
 
@@ -25,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     names = header_functions()
     assert len(names) >= 14
     for n in names:
-        assert hasattr(lib, n), f"{n} declared in include/dg_attn.h but not exported"
+        assert hasattr(lib, n), f"{n} declared in include/*.h but not exported"
     assert set(names) == set(capi.EXPORTS)
     assert lib.dg_attn_abi_version() == 1
 
