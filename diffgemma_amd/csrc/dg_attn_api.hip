@@ -68,6 +68,7 @@ struct Plan {
   uint32_t e_dtype = DG_BF16;   // element type the kernels compute in (bf16 or f16)
   bool convert_q = false, gather_kv = false, q_is_bf16 = false;
   bool scalar = false;
+  bool part_half = false;       // split partial rows travel as normalised f16 rows
   size_t off_q = 0, off_kv = 0, off_part_o = 0, off_part_ml = 0, total = 0;
   float scale = 1.0f;
 };
@@ -175,9 +176,12 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
     pl->off_kv = off;
     off += align_up((size_t)2 * d->n_kv_heads * pl->t_all * hd * 2);
   }
+  // f16 partial rows need |V| <= 65504: an f16 cache guarantees it, for a bf16 cache the caller says so
+  pl->part_half = pl->n_splits > 1 && d->out_dtype != DG_F32 && !(d->flags & DG_ATTN_F_F32_PARTIALS) &&
+                  (pl->e_dtype == DG_F16 || (d->flags & DG_ATTN_F_F16_PARTIALS));
   if (pl->n_splits > 1) {
     pl->off_part_o = off;
-    off += align_up((size_t)pl->n_splits * d->n_kv_heads * pl->rows_pad * hd * 4);
+    off += align_up((size_t)pl->n_splits * d->n_kv_heads * pl->rows_pad * hd * (pl->part_half ? 2 : 4));
     pl->off_part_ml = off;
     off += align_up((size_t)pl->n_splits * d->n_kv_heads * pl->rows_pad * 2 * 4);
   }
@@ -332,26 +336,18 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   p.q_is_bf16 = pl.q_is_bf16 ? 1u : 0u;
   p.out_dtype = d->out_dtype;
   p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
-  // f16 partial rows need |V| <= 65504: an f16 cache guarantees it, for a bf16 cache the caller says so
-  p.part_half = (pl.n_splits > 1 && d->out_dtype != DG_F32 && !(d->flags & DG_ATTN_F_F32_PARTIALS) &&
-                 (pl.e_dtype == DG_F16 || (d->flags & DG_ATTN_F_F16_PARTIALS)))
-                    ? 1u
-                    : 0u;
+  p.part_half = pl.part_half ? 1u : 0u;
   p.scale_log2 = pl.scale * dg::kLog2e;
   return DG_OK;
 }
 
 }  // namespace
 
-int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+namespace {
+// One attention call with its plan made: validation of the pointers, parameter block, launches.
+int forward_planned(const dg_attn_desc* d, const Plan& pl, const void* q, const void* kv_base, void* out, float* lse,
                     void* workspace, size_t workspace_bytes, void* stream) {
-  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
-  DeviceInfo di;
-  int rc = device_info(&di);
-  if (rc != DG_OK) return rc;
-  Plan pl;
-  rc = make_plan(d, di.cus, &pl);
-  if (rc != DG_OK) return rc;
+  int rc = DG_OK;
   if (pl.total > 0 && (!workspace || workspace_bytes < pl.total)) return DG_ERR_WORKSPACE;
   if (pl.total > 0 && ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
   if (((uintptr_t)q % 16) != 0 || ((uintptr_t)kv_base % 16) != 0 || ((uintptr_t)out % 16) != 0) return DG_ERR_LAYOUT;
@@ -381,6 +377,19 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
   }
   if (pl.n_splits > 1 && dg::launch_attn_merge(p, hd, s) != hipSuccess) return DG_ERR_LAUNCH;
   return DG_OK;
+}
+}  // namespace
+
+int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, di.cus, &pl);
+  if (rc != DG_OK) return rc;
+  return forward_planned(d, pl, q, kv_base, out, lse, workspace, workspace_bytes, stream);
 }
 
 namespace {
