@@ -105,8 +105,12 @@ def test_split_planning():
     assert capi.resolved_splits(A.make_desc(2, 4, 2, 32, 2)) == 1                 # one tile: nothing to split
     assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, n_splits=3)) == 3
     assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, kernel=capi.DG_KERNEL_SCALAR)) == 1
-    # workspace: 8 splits x 2 heads x 2048 rows x (512 + 2) floats
-    assert capi.workspace_bytes(W.config("cfg3_global").desc()) == 8 * 2 * 2048 * 514 * 4
+    # workspace: 8 splits x 2 heads x 2048 rows x (512 fp32 accumulators + (m, l)); the partial rows take
+    # half of that as f16 (the workload descriptors vouch for the range of V)
+    assert capi.workspace_bytes(W.config("cfg3_global").desc(flags=capi.DG_ATTN_F_F32_PARTIALS)) == 8 * 2 * 2048 * 514 * 4
+    assert capi.workspace_bytes(W.config("cfg3_global").desc()) == 8 * 2 * 2048 * (512 * 2 + 2 * 4)
+    assert capi.workspace_bytes(A.make_desc(256, 16, 2, 512, 32768)) == 8 * 2 * 2048 * 514 * 4                  # bf16 cache: fp32 unless asked
+    assert capi.workspace_bytes(A.make_desc(256, 16, 2, 512, 32768, kv_dtype=capi.DG_F16)) == 8 * 2 * 2048 * (512 * 2 + 2 * 4)
     assert capi.workspace_bytes(A.make_desc(2, 4, 2, 32, 2)) == 0
 
 
