@@ -24,6 +24,7 @@ DG_ROPE_F_QK_TRUNCATE = 0x1
 DG_OK = 0
 DG_ERR_NULL, DG_ERR_SHAPE, DG_ERR_DTYPE, DG_ERR_LAYOUT = -1, -2, -3, -4
 DG_ERR_WORKSPACE, DG_ERR_MASK, DG_ERR_LAUNCH, DG_ERR_DEVICE, DG_ERR_UNSUPPORTED = -5, -6, -7, -8, -9
+DG_ERR_SCRATCH_LIMIT = -10
 
 # every symbol include/*.h declares
 EXPORTS = (
@@ -36,6 +37,7 @@ EXPORTS = (
     "dg_attention_topk_dispatch", "dg_prof_end_split",
     "dg_kv_layer_reference_layout", "dg_kv_layer_head_major_layout", "dg_kv_snapshot_bytes", "dg_kv_snapshot_gather",
     "dg_kv_snapshot_scatter", "dg_kv_live_bytes", "dg_kv_live_gather", "dg_fnv1a64",
+    "dg_attn_forward_static", "dg_attn_static_scratch_bytes",
 )
 
 
@@ -137,6 +139,10 @@ def load():
     lib.dg_attn_resolved_splits.restype = C.c_int
     lib.dg_attn_forward.argtypes = [P(AttnDesc), VP, VP, VP, VP, VP, C.c_size_t, VP]
     lib.dg_attn_forward.restype = C.c_int
+    lib.dg_attn_forward_static.argtypes = [P(AttnDesc), VP, VP, VP, VP, VP]
+    lib.dg_attn_forward_static.restype = C.c_int
+    lib.dg_attn_static_scratch_bytes.argtypes = []
+    lib.dg_attn_static_scratch_bytes.restype = C.c_size_t
     lib.dg_attn_strerror.argtypes = [C.c_int]
     lib.dg_attn_strerror.restype = C.c_char_p
     lib.dg_attn_abi_version.argtypes = []

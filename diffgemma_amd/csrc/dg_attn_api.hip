@@ -25,6 +25,15 @@ struct DeviceInfo {
   int checked = 0;  // 0 unknown, 1 ok, -1 wrong arch
   int cus = 256;
 };
+
+// Device memory of dg_attn_forward_static, the entry point that may not allocate: what
+// dg_attn_forward takes as its workspace argument (split partial rows, converted copies of f32
+// inputs) lives here instead.  Every device the library runs on holds its own copy at its own
+// address until the process ends; the name below is only a host-side handle, the device address
+// is looked up once per device (static_scratch_ptr) and that pointer is what kernels are given.
+constexpr size_t kStaticScratchBytes = DG_ATTN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+void* g_scratch_ptr[64] = {};
 DeviceInfo g_dev[64];
 thread_local uint32_t* g_tls_dbg = nullptr;
 std::mutex g_dev_mu;
@@ -58,6 +67,20 @@ int device_info(DeviceInfo* out) {
 int plan_cus() {
   DeviceInfo di;
   return device_info(&di) == DG_OK ? di.cus : 256;
+}
+
+// Address of `scratch` on the current device, looked up the first time the device is seen.
+int static_scratch_ptr(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DG_ERR_DEVICE;
+  std::lock_guard<std::mutex> lock(g_dev_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return DG_ERR_DEVICE;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return DG_OK;
 }
 
 // Everything the launch needs that can be derived on the host without a device.
@@ -207,6 +230,9 @@ const char* dg_attn_strerror(int status) {
     case DG_ERR_LAUNCH: return "HIP launch failed";
     case DG_ERR_DEVICE: return "no gfx950 device current";
     case DG_ERR_UNSUPPORTED: return "request not implemented";
+    case DG_ERR_SCRATCH_LIMIT:
+      return "the call needs more scratch than dg_attn_forward_static holds (dg_attn_static_scratch_bytes); "
+             "use dg_attn_forward with a workspace";
     default: return "unknown status";
   }
 }
@@ -390,6 +416,26 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
   rc = make_plan(d, di.cus, &pl);
   if (rc != DG_OK) return rc;
   return forward_planned(d, pl, q, kv_base, out, lse, workspace, workspace_bytes, stream);
+}
+
+size_t dg_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int dg_attn_forward_static(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+                           void* stream) {
+  if (!d || !q || !kv_base || !out) return DG_ERR_NULL;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, di.cus, &pl);
+  if (rc != DG_OK) return rc;
+  if (pl.total > kStaticScratchBytes) return DG_ERR_SCRATCH_LIMIT;
+  void* ptr = nullptr;
+  rc = static_scratch_ptr(&ptr);
+  if (rc != DG_OK) return rc;
+  // Nothing in the scratch has to start at zero: a launch writes every partial row and every
+  // converted element it later reads.
+  return forward_planned(d, pl, q, kv_base, out, lse, ptr, kStaticScratchBytes, stream);
 }
 
 namespace {

@@ -43,7 +43,8 @@ typedef enum dg_status {
   DG_ERR_MASK = -6,        /* causal_rows > canvas, window/t_lo inconsistent */
   DG_ERR_LAUNCH = -7,      /* the HIP runtime refused a launch (sticky error text kept) */
   DG_ERR_DEVICE = -8,      /* not a gfx950 device, or no device */
-  DG_ERR_UNSUPPORTED = -9  /* valid request the library does not implement (e.g. q8 KV) */
+  DG_ERR_UNSUPPORTED = -9, /* valid request the library does not implement (e.g. q8 KV) */
+  DG_ERR_SCRATCH_LIMIT = -10 /* dg_attn_forward_static: the call needs more scratch than the library holds */
 } dg_status;
 
 typedef enum dg_dtype { DG_BF16 = 0, DG_F16 = 1, DG_F32 = 2 } dg_dtype;
@@ -119,6 +120,23 @@ int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits);
  * max(1e-3 |exact|, 2^-8). */
 int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* dg_attn_forward for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no workspace argument.  It has no
+ * counterpart in the reference.  The scratch dg_attn_forward takes from its workspace (split
+ * partial rows, converted copies of f32 inputs) lives in DG_ATTN_STATIC_SCRATCH_BYTES of device
+ * memory inside the library, held on every GPU the library runs on until the process ends; a call
+ * whose dg_attn_workspace_bytes() exceeds that returns DG_ERR_SCRATCH_LIMIT and enqueues nothing.
+ * 40 MiB covers the model's layers with f16 partial rows (global layer at any prefix: 32.3 MiB;
+ * a 1024-row prefill super-chunk: 32.3 MiB), not a global layer with fp32 partial rows (64.3 MiB).
+ * Same kernels, same results as dg_attn_forward, bit for bit.  The call allocates and frees
+ * nothing; its first call on a device looks the scratch address up (do that once outside a graph
+ * capture).  All calls on one GPU share the one scratch: calls that overlap on a GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe. */
+#define DG_ATTN_STATIC_SCRATCH_BYTES (40u << 20)
+int dg_attn_forward_static(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
+                           void* stream);
+size_t dg_attn_static_scratch_bytes(void);
 
 const char* dg_attn_strerror(int status);
 uint32_t dg_attn_abi_version(void);
