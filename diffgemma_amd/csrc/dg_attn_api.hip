@@ -109,6 +109,8 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
     return DG_ERR_SHAPE;
   }
   if ((uint64_t)d->kv_len + d->canvas > 0x7fffffffull) return DG_ERR_SHAPE;
+  // the kernels address query rows with 32-bit byte offsets
+  if ((uint64_t)d->canvas * d->n_q_heads * hd * 2ull >= (1ull << 32)) return DG_ERR_SHAPE;
   if (d->q_dtype > DG_F32 || d->kv_dtype > DG_F32 || d->out_dtype > DG_F32) return DG_ERR_DTYPE;
   if (d->out_dtype == DG_F16) return DG_ERR_DTYPE;
   if (d->causal_rows > d->canvas) return DG_ERR_MASK;

@@ -62,6 +62,8 @@ def test_descriptor_validation_codes():
     assert _status(A.make_desc(256, 16, 2, 96, 1024)) == capi.DG_ERR_SHAPE         # head_dim
     assert _status(A.make_desc(0, 16, 2, 512, 1024)) == capi.DG_ERR_SHAPE          # empty canvas
     assert _status(A.make_desc(256, 16, 3, 512, 1024)) == capi.DG_ERR_SHAPE        # Hq % Hkv
+    assert _status(A.make_desc(65536, 128, 2, 512, 1024)) == capi.DG_ERR_SHAPE     # query rows past 4 GiB (32-bit row offsets)
+    assert _status(A.make_desc(65536, 32, 2, 512, 1024)) == capi.DG_OK
     assert _status(A.make_desc(256, 16, 2, 512, 1024, causal_rows=257)) == capi.DG_ERR_MASK
     assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_ring_mask=1000)) == capi.DG_ERR_LAYOUT
     assert _status(A.make_desc(256, 16, 2, 512, 1024, kv_ring_mask=15)) == capi.DG_ERR_LAYOUT  # ring < key tile
