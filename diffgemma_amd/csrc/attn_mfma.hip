@@ -104,6 +104,20 @@ __device__ __forceinline__ void scale_acc4(float& x0, float& x1, float& x2, floa
       : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
       : "v"(c));
 }
+// Four values out of accumulation registers.  Spelled out so that the epilogue takes O from where
+// the tile loop left it, a few registers at a time: left to itself the compiler moves all of O
+// into VGPRs at the loop's exit, runs out of them and parks part of O in scratch memory, and the
+// reloads then queue behind the epilogue's own stores (one memory counter serves both), which
+// made every 32-row block wait for the previous block's stores to complete.
+template <bool FROM_ACC>
+__device__ __forceinline__ f32x4 acc_read4(const f32x16& a, int e) {
+  if constexpr (!FROM_ACC) return f32x4{a[e], a[e + 1], a[e + 2], a[e + 3]};   // smaller head_dim: O does not fill the registers
+  float t0, t1, t2, t3;
+  asm volatile("v_accvgpr_read_b32 %0, %4\n\tv_accvgpr_read_b32 %1, %5\n\tv_accvgpr_read_b32 %2, %6\n\tv_accvgpr_read_b32 %3, %7"
+               : "=v"(t0), "=v"(t1), "=v"(t2), "=v"(t3)
+               : "a"(a[e]), "a"(a[e + 1]), "a"(a[e + 2]), "a"(a[e + 3]));
+  return f32x4{t0, t1, t2, t3};
+}
 // dst = src for a score tile, as instructions the compiler cannot move or merge away; part I of
 // 8 copies elements 2 I and 2 I + 1
 template <int I>
@@ -654,9 +668,10 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         const f32x16& a = o[i * NRBW + j];
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4 x = acc_read4<D == 512>(a, 4 * q4);
           u32x2 h2;
-          h2[0] = pack2<true>(sat_f16(a[4 * q4] * inv), sat_f16(a[4 * q4 + 1] * inv));
-          h2[1] = pack2<true>(sat_f16(a[4 * q4 + 2] * inv), sat_f16(a[4 * q4 + 3] * inv));
+          h2[0] = pack2<true>(sat_f16(x[0] * inv), sat_f16(x[1] * inv));
+          h2[1] = pack2<true>(sat_f16(x[2] * inv), sat_f16(x[3] * inv));
           *(__attribute__((address_space(3))) u32x2*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 2) = h2;
         }
       }
@@ -683,7 +698,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         const f32x16& a = o[i * NRBW + j];
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
-          f32x4 v4 = {a[4 * q4], a[4 * q4 + 1], a[4 * q4 + 2], a[4 * q4 + 3]};
+          const f32x4 v4 = acc_read4<D == 512>(a, 4 * q4);
           *(__attribute__((address_space(3))) f32x4*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 4) = v4;
         }
       }
@@ -707,8 +722,9 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const f32x16& a = o[i * NRBW + j];
-        const float y0 = a[4 * q4] * inv, y1 = a[4 * q4 + 1] * inv;
-        const float y2 = a[4 * q4 + 2] * inv, y3 = a[4 * q4 + 3] * inv;
+        const f32x4 x = acc_read4<D == 512>(a, 4 * q4);
+        const float y0 = x[0] * inv, y1 = x[1] * inv;
+        const float y2 = x[2] * inv, y3 = x[3] * inv;
         const size_t idx = idx0 + 8 * q4;
         if (p.dbg && !(fabsf(y0) + fabsf(y1) + fabsf(y2) + fabsf(y3) <= 3.402823466e38f))   // NaN or infinity
           dbg_report(p.dbg, 2u, (tok_o << 16) | qh_o, 32u * (dgrp * NDBW + i) + 4u * g2 + 8u * q4);
