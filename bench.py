@@ -80,7 +80,8 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
 # WRITE_SIZE counters of rocprofv3, each scaled by what the same counter reads for the
 # calibration copy (--calib-copy-mib): fetch x2.000, write x1.000.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "cfg3_global": (161.1e6 + 42.5e6, "profiles/attn_mfma_kernel_cfg3_global_hbm_traffic.md"),
+    "cfg3_global": (152.5e6 + 33.8e6, "profiles/attn_mfma_kernel_cfg3_global_hbm_traffic.md"),
+    "cfg4_long": (555.3e6 + 33.8e6, "profiles/attn_mfma_kernel_cfg4_long_hbm_traffic.md"),
 }
 
 
@@ -683,7 +684,10 @@ def main():
                      "frac_of_mfma_only_microkernel": kern_tflops / mfma_only_tflops,
                      "mfma_only_random_operands_tflops": mfma_random_tflops,
                      "frac_of_mfma_only_random_operands": kern_tflops / mfma_random_tflops,
-                     "kv_gbs": kv_bytes / (kern_ms * 1e-3) / 1e9, "hbm_peak_gbs": PEAK_HBM_GBS},
+                     "kv_gbs": kv_bytes / (kern_ms * 1e-3) / 1e9,
+                     # achieved HBM bandwidth of the kernel: the profiled bytes per launch over this run's kernel time
+                     "hbm_gbs": traffic / (kern_ms * 1e-3) / 1e9 if traffic else None,
+                     "hbm_peak_gbs": PEAK_HBM_GBS},
         "rounds": rounds, "settle": settle, "check": check, "input_gen_s": t_gen,
     }
     if not args.no_cpu_baseline:
