@@ -194,6 +194,45 @@ def forward(desc: capi.AttnDesc, q, kv, out, lse=None, workspace=None) -> None:
                                    lse.data_ptr() if lse is not None else None, ws_ptr, ws_bytes, stream_handle()))
 
 
+def state_bytes(desc: capi.AttnDesc) -> int:
+    n = C.c_size_t(0)
+    capi.check(capi.load().dg_attn_state_bytes(C.byref(desc), C.byref(n)))
+    return n.value
+
+
+def alloc_state(desc: capi.AttnDesc):
+    """Device memory for one attention state (m, l, acc) of `desc`."""
+    return _torch().empty(state_bytes(desc), dtype=_torch().uint8, device="cuda")
+
+
+def partial(desc: capi.AttnDesc, t_begin: int, t_end: int, q, kv, state) -> None:
+    """State of the keys [t_begin, t_end) under desc's mask (dg_attn_partial); the workspace is made here."""
+    torch = _torch()
+    n = C.c_size_t(0)
+    lib = capi.load()
+    capi.check(lib.dg_attn_partial_workspace_bytes(C.byref(desc), t_begin, t_end, C.byref(n)))
+    ws = torch.empty(max(n.value, 256), dtype=torch.uint8, device="cuda")
+    capi.check(lib.dg_attn_partial(C.byref(desc), t_begin, t_end, q.data_ptr(), kv.data_ptr(), state.data_ptr(),
+                                   state.numel(), ws.data_ptr(), ws.numel(), stream_handle()))
+    torch.cuda.current_stream().synchronize()   # ws is released on return
+
+
+def merge(desc: capi.AttnDesc, states, out=None, lse=None, state_out=None) -> None:
+    """dg_attn_merge of a list of states into out (+ lse) and/or a state."""
+    arr = (C.c_void_p * len(states))(*[s.data_ptr() for s in states])
+    capi.check(capi.load().dg_attn_merge(C.byref(desc), arr, len(states), out.data_ptr() if out is not None else None,
+                                         lse.data_ptr() if lse is not None else None,
+                                         state_out.data_ptr() if state_out is not None else None, stream_handle()))
+
+
+def read_state(desc: capi.AttnDesc, state):
+    """(m [rows], l [rows], acc [rows, hd]) of a state, rows = canvas * n_q_heads, as numpy arrays."""
+    rows = desc.canvas * desc.n_q_heads
+    f = state.cpu().numpy().view(np.float32)
+    off = (2 * rows + 3) & ~3
+    return f[:rows].copy(), f[rows:2 * rows].copy(), f[off:off + rows * desc.head_dim].reshape(rows, desc.head_dim).copy()
+
+
 def alloc_workspace(desc: capi.AttnDesc):
     torch = _torch()
     n = capi.workspace_bytes(desc)

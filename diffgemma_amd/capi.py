@@ -38,6 +38,8 @@ EXPORTS = (
     "dg_kv_layer_reference_layout", "dg_kv_layer_head_major_layout", "dg_kv_snapshot_bytes", "dg_kv_snapshot_gather",
     "dg_kv_snapshot_scatter", "dg_kv_live_bytes", "dg_kv_live_gather", "dg_fnv1a64",
     "dg_attn_forward_static", "dg_attn_static_scratch_bytes",
+    "dg_attn_state_bytes", "dg_attn_partial_workspace_bytes", "dg_attn_partial", "dg_attn_merge",
+    "dg_attention_dispatch_block", "dg_attention_block_state_bytes",
 )
 
 
@@ -154,6 +156,19 @@ def load():
     lib.dg_attention_dispatch.restype = C.c_int
     lib.dg_attention_state_bytes.argtypes = [P(LayerOffsets), P(AttnDims), C.c_uint32, P(C.c_size_t)]
     lib.dg_attention_state_bytes.restype = C.c_int
+    lib.dg_attention_dispatch_block.argtypes = [VP, VP, VP, P(LayerOffsets), P(StepParams), P(AttnDims),
+                                                P(AttnBlockRange), VP, VP, C.c_size_t, VP]
+    lib.dg_attention_dispatch_block.restype = C.c_int
+    lib.dg_attention_block_state_bytes.argtypes = [P(LayerOffsets), P(AttnDims), C.c_uint32, P(C.c_size_t)]
+    lib.dg_attention_block_state_bytes.restype = C.c_int
+    lib.dg_attn_state_bytes.argtypes = [P(AttnDesc), P(C.c_size_t)]
+    lib.dg_attn_state_bytes.restype = C.c_int
+    lib.dg_attn_partial_workspace_bytes.argtypes = [P(AttnDesc), C.c_uint32, C.c_uint32, P(C.c_size_t)]
+    lib.dg_attn_partial_workspace_bytes.restype = C.c_int
+    lib.dg_attn_partial.argtypes = [P(AttnDesc), C.c_uint32, C.c_uint32, VP, VP, VP, C.c_size_t, VP, C.c_size_t, VP]
+    lib.dg_attn_partial.restype = C.c_int
+    lib.dg_attn_merge.argtypes = [P(AttnDesc), P(VP), C.c_uint32, VP, VP, VP, VP]
+    lib.dg_attn_merge.restype = C.c_int
     lib.dg_kv_row_bytes.argtypes = [C.c_uint32, C.c_uint32]
     lib.dg_kv_row_bytes.restype = C.c_uint64
     lib.dg_kv_region_bytes.argtypes = [C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32]

@@ -60,9 +60,9 @@ __global__ void __launch_bounds__(64) attn_scalar_kernel(const AttnParams p, con
     }
   }
   float m = -INFINITY, l = 0.f;
-  for (uint32_t t = b.lo; t < p.t_all; ++t) {
-    if (!key_visible(b, t, p.t_all)) {
-      if (t >= b.hi && b.extra >= p.t_all) break;
+  for (uint32_t t = b.lo; t < p.t_clip_hi; ++t) {
+    if (!key_visible(b, t, p.t_clip_hi)) {
+      if (t >= b.hi && b.extra >= p.t_clip_hi) break;
       continue;
     }
     const int64_t slot = kv_slot(p.ring_mask, t);
@@ -382,6 +382,83 @@ hipError_t launch_attn_scalar(const AttnParams& p, uint32_t head_dim, uint32_t k
     hipLaunchKernelGGL(attn_scalar_kernel<uint16_t>, grid, block, 0, s, p, head_dim);
   else
     hipLaunchKernelGGL(attn_scalar_kernel<_Float16>, grid, block, 0, s, p, head_dim);
+  return hipGetLastError();
+}
+
+// One wave per (canvas row, query head): the closed form  m = max m_i,  l = sum l_i e^(m_i - m),
+// acc = sum acc_i e^(m_i - m)  over the states that saw a key, written as the final row (acc / l)
+// and/or as a state again, in the normal form (m + ln l, 1, acc / l).
+__global__ void __launch_bounds__(256) attn_state_merge_kernel(const StateMergeParams p) {
+  const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * 4 + wave;
+  if (row >= p.rows) return;
+  float mx = -INFINITY;
+  for (uint32_t i = 0; i < p.n; ++i) {
+    const float2 ml = make_float2(p.states[i][row], p.states[i][p.rows + row]);
+    if (ml.y > 0.f) mx = fmaxf(mx, ml.x);
+  }
+  float den = 0.f;
+  for (uint32_t i = 0; i < p.n; ++i) {
+    const float2 ml = make_float2(p.states[i][row], p.states[i][p.rows + row]);
+    if (ml.y > 0.f) den += ml.y * __expf(ml.x - mx);
+  }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  const size_t acc0 = state_acc_offset(p.rows) + (size_t)row * p.hd;
+  for (uint32_t d = lane * 4u; d < p.hd; d += 256u) {
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t i = 0; i < p.n; ++i) {
+      const float2 ml = make_float2(p.states[i][row], p.states[i][p.rows + row]);
+      if (!(ml.y > 0.f)) continue;
+      const float w = __expf(ml.x - mx);
+      const float4 a = *(const float4*)(p.states[i] + acc0 + d);
+      o.x = __builtin_fmaf(w, a.x, o.x);
+      o.y = __builtin_fmaf(w, a.y, o.y);
+      o.z = __builtin_fmaf(w, a.z, o.z);
+      o.w = __builtin_fmaf(w, a.w, o.w);
+    }
+    o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
+    if (p.dbg && (nonfinite(o.x) || nonfinite(o.y) || nonfinite(o.z) || nonfinite(o.w)))
+      dbg_report(p.dbg, 2u, ((row / p.hq) << 16) | (row % p.hq), d);
+    if (p.state_out) *(float4*)(p.state_out + acc0 + d) = o;
+    if (p.out) {
+      const size_t idx = (size_t)row * p.hd + d;
+      if (p.out_dtype == DT_F32) {
+        *(float4*)((float*)p.out + idx) = o;
+      } else if (p.out_dtype == DT_BF16) {
+        const bool tr = p.out_trunc != 0;
+        uint2 pk;
+        pk.x = (uint32_t)f32_to_bf16_bits(o.x, tr) | ((uint32_t)f32_to_bf16_bits(o.y, tr) << 16);
+        pk.y = (uint32_t)f32_to_bf16_bits(o.z, tr) | ((uint32_t)f32_to_bf16_bits(o.w, tr) << 16);
+        *(uint2*)((uint16_t*)p.out + idx) = pk;
+      } else {
+        _Float16* const h = (_Float16*)p.out + idx;
+        h[0] = (_Float16)o.x; h[1] = (_Float16)o.y; h[2] = (_Float16)o.z; h[3] = (_Float16)o.w;
+      }
+    }
+  }
+  if (lane == 0) {
+    const float lse = den > 0.f ? mx + __logf(den) : -INFINITY;
+    if (p.dbg && p.out && !(den > 0.f)) dbg_report(p.dbg, 1u, ((row / p.hq) << 16) | (row % p.hq), __float_as_uint(den));
+    if (p.lse) p.lse[row] = lse;
+    if (p.state_out) {
+      p.state_out[row] = lse;
+      p.state_out[p.rows + row] = den > 0.f ? 1.f : 0.f;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) state_unit_l_kernel(const float* m_plane, float* l_plane, uint32_t rows) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i < rows) l_plane[i] = m_plane[i] == -INFINITY ? 0.f : 1.f;   // (a NaN stays visible: l = 1)
+}
+
+hipError_t launch_state_unit_l(float* m_plane, float* l_plane, uint32_t rows, hipStream_t s) {
+  hipLaunchKernelGGL(state_unit_l_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, m_plane, l_plane, rows);
+  return hipGetLastError();
+}
+
+hipError_t launch_state_merge(const StateMergeParams& p, hipStream_t s) {
+  hipLaunchKernelGGL(attn_state_merge_kernel, dim3((p.rows + 3) / 4), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 

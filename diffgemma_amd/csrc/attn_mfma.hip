@@ -233,7 +233,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       hi_min = min(hi_min, min(bc.hi, bd.hi));
       hi_max = max(hi_max, max(bc.hi, bd.hi));
     }
-    if (tok_a < p.causal_rows && p.extra_lo < p.t_all) hi_max = p.t_all;
+    if (tok_a < p.causal_rows && p.extra_lo < p.t_clip_hi) hi_max = p.t_clip_hi;
     if (row0 + kBlockM > p.rows_total) hi_min = 0;  // ragged tile: always take the masked path
     // all four are the same in every lane; say so, so that they live in scalar registers
     lo_min = __builtin_amdgcn_readfirstlane(lo_min);
@@ -401,7 +401,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const uint32_t t = t0 + 8u * (e >> 2) + 4u * g2 + (e & 3);
-            if (!key_visible(rb, t, p.t_all)) s[e] = -INFINITY;
+            if (!key_visible(rb, t, p.t_clip_hi)) s[e] = -INFINITY;
           }
         }
       } else if constexpr (c == 1) {

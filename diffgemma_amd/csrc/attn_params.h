@@ -34,6 +34,7 @@ struct AttnParams {
   uint32_t lo_nc;        // first visible key of a non-causal row
   uint32_t extra_lo;     // causal rows also see keys >= extra_lo (t_all = none)
   uint32_t ring_mask;
+  uint32_t t_clip_lo, t_clip_hi;   // only keys in [t_clip_lo, t_clip_hi) count (a key-range partial); the whole range: 0, t_all
   uint32_t rows_total, rows_pad, n_mtiles;
   uint32_t n_splits, tile_first, tiles_per_split, tile_end;
   uint32_t q_is_bf16;    // Q holds bf16 although E is f16 (reference: bf16 activations, f16 cache)
@@ -56,6 +57,22 @@ struct TopkParams {
   float scale;
 };
 
+// Merging attention states of key-range partials (dg_attn_merge).  A state holds, per row
+// (row = canvas row * n_q_heads + query head), m and l in two planes of `rows` floats and then, from
+// the next 16-byte boundary, head_dim accumulators `acc` per row, with
+//   output row = acc / l,   log-sum-exp of the row's scores = m + ln l   (natural log; l = 0: no key seen).
+constexpr uint32_t kMaxStates = 16;
+__host__ __device__ inline size_t state_acc_offset(size_t rows) { return (2 * rows + 3) & ~(size_t)3; }   // floats
+struct StateMergeParams {
+  const float* states[kMaxStates];
+  uint32_t n, rows, hd, hq;
+  void* out;            // [rows][head_dim] of out_dtype, or null
+  float* lse;           // [rows] or null
+  float* state_out;     // a state, or null; may be one of `states` (a row is read before it is written)
+  uint32_t out_dtype, out_trunc;
+  uint32_t* dbg;
+};
+
 struct RowBounds {
   uint32_t lo, hi, extra;  // visible iff (lo <= t < hi) or (extra <= t), and t < t_all
 };
@@ -75,6 +92,9 @@ __device__ __forceinline__ RowBounds row_bounds(const AttnParams& p, uint32_t to
     b.lo = p.lo_nc;
     b.extra = p.t_all;
   }
+  b.lo = max(b.lo, p.t_clip_lo);
+  b.hi = min(b.hi, p.t_clip_hi);
+  b.extra = max(b.extra, p.t_clip_lo);   // (keys at or past t_clip_hi are cut by key_visible's last argument)
   return b;
 }
 
@@ -113,6 +133,9 @@ __device__ __forceinline__ void dbg_report(uint32_t* dbg, uint32_t code, uint32_
 hipError_t launch_attn_scalar(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 hipError_t launch_attn_mfma(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, hipStream_t s);
+hipError_t launch_state_merge(const StateMergeParams& p, hipStream_t s);
+// l[row] = 1 where m[row] is finite, else 0: completes a state whose rows are already normalised
+hipError_t launch_state_unit_l(float* m_plane, float* l_plane, uint32_t rows, hipStream_t s);
 hipError_t launch_convert(const void* src, uint32_t src_dtype, void* dst, uint32_t dst_dtype, size_t n, hipStream_t s);
 // gathers keys [0,t_all) of a strided (possibly ring) cache into planes [hkv][t_all][D] of dst_dtype
 hipError_t launch_kv_gather(const void* src, uint32_t src_dtype, void* dst, uint32_t dst_dtype, uint32_t hkv,

@@ -87,6 +87,7 @@ int static_scratch_ptr(void** out) {
 struct Plan {
   uint32_t group = 0, rows_total = 0, n_mtiles = 0, rows_pad = 0;
   uint32_t t_all = 0, lo_nc = 0, extra_lo = 0, win_m1 = 0xffffffffu;
+  uint32_t clip_lo = 0, clip_hi = 0;   // keys that count: [clip_lo, clip_hi); the whole range unless a partial is asked for
   uint32_t tile_first = 0, tile_end = 0, tiles_per_split = 0, n_splits = 1;
   uint32_t e_dtype = DG_BF16;   // element type the kernels compute in (bf16 or f16)
   bool convert_q = false, gather_kv = false, q_is_bf16 = false;
@@ -96,7 +97,7 @@ struct Plan {
   float scale = 1.0f;
 };
 
-int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
+int make_plan(const dg_attn_desc* d, int cus, Plan* pl, const uint32_t* key_range = nullptr) {
   if (!d) return DG_ERR_NULL;
   const uint32_t hd = d->head_dim;
   if (d->canvas == 0 || d->canvas > 65536 || d->n_q_heads == 0 || d->n_kv_heads == 0) return DG_ERR_SHAPE;
@@ -172,8 +173,16 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl) {
   lo_all = std::min(lo_all, pl->t_all);
   // a ring must hold every visible position at once, or two of them share a slot
   if (d->kv_ring_mask != 0 && pl->t_all - lo_all > d->kv_ring_mask + 1u) return DG_ERR_LAYOUT;
+  pl->clip_lo = 0;
+  pl->clip_hi = pl->t_all;
+  if (key_range) {
+    if (key_range[0] > key_range[1]) return DG_ERR_MASK;
+    pl->clip_lo = std::min(key_range[0], pl->t_all);
+    pl->clip_hi = std::min(key_range[1], pl->t_all);
+    lo_all = std::max(lo_all, pl->clip_lo);
+  }
   pl->tile_first = lo_all / dg::kBlockN;
-  pl->tile_end = (pl->t_all + dg::kBlockN - 1) / dg::kBlockN;
+  pl->tile_end = std::max(pl->tile_first, (pl->clip_hi + dg::kBlockN - 1) / dg::kBlockN);
   const uint32_t ntiles = std::max(1u, pl->tile_end - pl->tile_first);
 
   uint32_t splits = d->n_splits;
@@ -314,6 +323,8 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   const char* region = (const char*)kv_base + d->kv_region_bytes;
   p.q = q;
   p.ring_mask = d->kv_ring_mask;
+  p.t_clip_lo = pl.clip_lo;
+  p.t_clip_hi = pl.clip_hi;
   if (pl.convert_q) {
     if (dg::launch_convert(q, d->q_dtype, ws + pl.off_q, DG_BF16, (size_t)d->canvas * d->n_q_heads * hd, s) != hipSuccess)
       return DG_ERR_LAUNCH;
@@ -438,6 +449,97 @@ int dg_attn_forward_static(const dg_attn_desc* d, const void* q, const void* kv_
   // Nothing in the scratch has to start at zero: a launch writes every partial row and every
   // converted element it later reads.
   return forward_planned(d, pl, q, kv_base, out, lse, ptr, kStaticScratchBytes, stream);
+}
+
+// ---- key-range partials and their merge --------------------------------------------------------
+
+namespace {
+inline size_t state_bytes_of(const dg_attn_desc* d) {
+  const size_t rows = (size_t)d->canvas * d->n_q_heads;
+  return (dg::state_acc_offset(rows) + rows * d->head_dim) * sizeof(float);
+}
+// The descriptor of a partial: the caller's, with an fp32 result (the state's accumulators).
+inline dg_attn_desc partial_desc(const dg_attn_desc* d) {
+  dg_attn_desc pd = *d;
+  pd.out_dtype = DG_F32;
+  pd.flags &= ~(uint32_t)(DG_ATTN_F_OUT_TRUNCATE | DG_ATTN_F_F16_PARTIALS);
+  return pd;
+}
+}  // namespace
+
+int dg_attn_state_bytes(const dg_attn_desc* d, size_t* out_bytes) {
+  if (!d || !out_bytes) return DG_ERR_NULL;
+  Plan pl;
+  const int rc = make_plan(d, plan_cus(), &pl);
+  if (rc != DG_OK) return rc;
+  *out_bytes = state_bytes_of(d);
+  return DG_OK;
+}
+
+int dg_attn_partial_workspace_bytes(const dg_attn_desc* d, uint32_t t_begin, uint32_t t_end, size_t* out_bytes) {
+  if (!d || !out_bytes) return DG_ERR_NULL;
+  const dg_attn_desc pd = partial_desc(d);
+  const uint32_t range[2] = {t_begin, t_end};
+  Plan pl;
+  const int rc = make_plan(&pd, plan_cus(), &pl, range);
+  if (rc != DG_OK) return rc;
+  *out_bytes = pl.total;
+  return DG_OK;
+}
+
+int dg_attn_partial(const dg_attn_desc* d, uint32_t t_begin, uint32_t t_end, const void* q, const void* kv_base,
+                    void* state, size_t state_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d || !q || !kv_base || !state) return DG_ERR_NULL;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  const dg_attn_desc pd = partial_desc(d);
+  const uint32_t range[2] = {t_begin, t_end};
+  Plan pl;
+  rc = make_plan(&pd, di.cus, &pl, range);
+  if (rc != DG_OK) return rc;
+  if (state_bytes < state_bytes_of(d) || ((uintptr_t)state % 16) != 0) return DG_ERR_WORKSPACE;
+  // The attention kernels leave the row normalised (acc / l) and its log-sum-exp: the state's normal
+  // form is exactly that, (m, l) = (lse, 1), or (-inf, 0) for a row that saw no key of the range.
+  const size_t rows = (size_t)d->canvas * d->n_q_heads;
+  float* const m_plane = (float*)state;
+  float* const acc = m_plane + dg::state_acc_offset(rows);
+  rc = forward_planned(&pd, pl, q, kv_base, acc, m_plane, workspace, workspace_bytes, stream);
+  if (rc != DG_OK) return rc;
+  return dg::launch_state_unit_l(m_plane, m_plane + rows, (uint32_t)rows, (hipStream_t)stream) == hipSuccess
+             ? DG_OK
+             : DG_ERR_LAUNCH;
+}
+
+int dg_attn_merge(const dg_attn_desc* d, const void* const* states, uint32_t n_states, void* out, float* lse,
+                  void* state_out, void* stream) {
+  if (!d || !states) return DG_ERR_NULL;
+  if (!out && !state_out) return DG_ERR_NULL;
+  if (n_states == 0 || n_states > dg::kMaxStates) return DG_ERR_SHAPE;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, di.cus, &pl);
+  if (rc != DG_OK) return rc;
+  dg::StateMergeParams p;
+  std::memset(&p, 0, sizeof(p));
+  for (uint32_t i = 0; i < n_states; ++i) {
+    if (!states[i] || ((uintptr_t)states[i] % 16) != 0) return DG_ERR_NULL;
+    p.states[i] = (const float*)states[i];
+  }
+  if ((out && ((uintptr_t)out % 16) != 0) || (state_out && ((uintptr_t)state_out % 16) != 0)) return DG_ERR_LAYOUT;
+  p.n = n_states;
+  p.rows = d->canvas * d->n_q_heads;
+  p.hd = d->head_dim;
+  p.hq = d->n_q_heads;
+  p.out = out;
+  p.lse = lse;
+  p.state_out = (float*)state_out;
+  p.out_dtype = d->out_dtype;
+  p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
+  p.dbg = g_tls_dbg;
+  return dg::launch_state_merge(p, (hipStream_t)stream) == hipSuccess ? DG_OK : DG_ERR_LAUNCH;
 }
 
 namespace {
@@ -574,6 +676,50 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
   desc_from_reference(L, dims, P->kv_len, &d);
   g_tls_dbg = (uint32_t*)dbg;
   const int rc = dg_attn_forward(&d, q, kvcache, out, nullptr, attn_state, attn_state_bytes, stream);
+  g_tls_dbg = nullptr;
+  return rc;
+}
+
+int dg_attention_block_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                                   size_t* out_bytes) {
+  if (!L || !dims || !out_bytes) return DG_ERR_NULL;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, kv_len, &d);
+  size_t ws_full = 0, ws_part = 0;
+  int rc = dg_attn_workspace_bytes(&d, &ws_full);
+  if (rc != DG_OK) return rc;
+  // a block's partial never needs more than the partial of the whole range (fewer key tiles: fewer splits)
+  rc = dg_attn_partial_workspace_bytes(&d, 0u, d.kv_len + d.canvas, &ws_part);
+  if (rc != DG_OK) return rc;
+  *out_bytes = 2 * align_up(state_bytes_of(&d)) + std::max(ws_full, ws_part);
+  return DG_OK;
+}
+
+int dg_attention_dispatch_block(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                                const dg_step_params* P, const dg_attn_dims* dims, const dg_attn_block_range* blk,
+                                dg_debug_status* dbg, void* attn_state, size_t attn_state_bytes, void* stream) {
+  if (!L || !P || !dims || !blk) return DG_ERR_NULL;
+  if (blk->is_first && blk->is_last)
+    return dg_attention_dispatch(q, kvcache, out, L, P, dims, dbg, attn_state, attn_state_bytes, stream);
+  if (!attn_state || ((uintptr_t)attn_state % 16) != 0) return DG_ERR_WORKSPACE;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, P->kv_len, &d);
+  const size_t sb = align_up(state_bytes_of(&d));
+  if (attn_state_bytes < 2 * sb) return DG_ERR_WORKSPACE;
+  char* const carried = (char*)attn_state;        // (m, l, acc) of the blocks so far
+  char* const fresh = carried + sb;               // this block's own partial
+  char* const ws = carried + 2 * sb;
+  const size_t ws_bytes = attn_state_bytes - 2 * sb;
+  // A block with no key for some rows (a causal row's range ends before it) leaves l = 0 there, and
+  // the merge passes the carried state through, which is what the reference's early return does.
+  int rc = dg_attn_partial(&d, blk->t_begin, blk->t_end, q, kvcache, blk->is_first ? carried : fresh, sb, ws, ws_bytes,
+                           stream);
+  if (rc != DG_OK || blk->is_first) return rc;
+  const void* both[2] = {carried, fresh};
+  if (!blk->is_last) return dg_attn_merge(&d, both, 2u, nullptr, nullptr, carried, stream);
+  if (!out) return DG_ERR_NULL;
+  g_tls_dbg = (uint32_t*)dbg;
+  rc = dg_attn_merge(&d, both, 2u, out, nullptr, nullptr, stream);
   g_tls_dbg = nullptr;
   return rc;
 }

@@ -138,6 +138,37 @@ int dg_attn_forward_static(const dg_attn_desc* d, const void* q, const void* kv_
                            void* stream);
 size_t dg_attn_static_scratch_bytes(void);
 
+/* ---- key-range partials and their merge ----
+ *
+ * The reference's attention_mma_full can be dispatched once per block of keys, in order, with the
+ * softmax state (m, l, unnormalised O) carried in attn_state between the dispatches
+ * (src/shaders/attn/attention/attention_mma_full.metal:107-118 state planes, 151-186 resume,
+ * 355-368 persist; host loop src/metal/step_kernel/enc.rs:2261-2291).  The same split is the
+ * key-length sharding of this path over devices: each holder of a key range produces a state,
+ * one exchange later any of them merges.  Two calls expose it:
+ *
+ * dg_attn_partial attends only the keys t_begin <= t < t_end (positions in the mask's numbering:
+ * prefix keys 0 .. kv_len-1, canvas keys kv_len ..; the range may be empty, may end past the last
+ * key and need not be aligned) under the descriptor's mask, and writes a state.
+ * dg_attn_merge combines 1 .. 16 states of the same descriptor into the output rows (out, in the
+ * descriptor's out_dtype and rounding, with lse if not NULL) and/or into a state again (state_out,
+ * which may be one of the inputs).  Merging the partials of ranges that tile [0, kv_len + canvas)
+ * gives dg_attn_forward's result up to fp32 rounding, whatever the cuts.
+ *
+ * A state is device memory of dg_attn_state_bytes(): with rows = canvas * n_q_heads and
+ * row = canvas_row * n_q_heads + head: float m[rows], float l[rows], then from the next 16-byte
+ * boundary float acc[rows][head_dim]; output row = acc / l, log-sum-exp = m + ln l (natural log),
+ * l = 0 for a row that saw no key.  (The reference keeps the same three quantities head-major;
+ * nothing outside the kernels reads its planes.)  dg_attn_partial leaves states in the normal
+ * form l = 1, acc = the normalised row.  The workspace of a partial is sized by
+ * dg_attn_partial_workspace_bytes for the same range. */
+int dg_attn_state_bytes(const dg_attn_desc* d, size_t* out_bytes);
+int dg_attn_partial_workspace_bytes(const dg_attn_desc* d, uint32_t t_begin, uint32_t t_end, size_t* out_bytes);
+int dg_attn_partial(const dg_attn_desc* d, uint32_t t_begin, uint32_t t_end, const void* q, const void* kv_base,
+                    void* state, size_t state_bytes, void* workspace, size_t workspace_bytes, void* stream);
+int dg_attn_merge(const dg_attn_desc* d, const void* const* states, uint32_t n_states, void* out, float* lse,
+                  void* state_out, void* stream);
+
 const char* dg_attn_strerror(int status);
 uint32_t dg_attn_abi_version(void);
 /* Visible (row,key) pairs per head and the FLOP count 4*head_dim*n_q_heads*pairs
@@ -192,6 +223,20 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
                           void* attn_state, size_t attn_state_bytes, void* stream);
 int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
                              size_t* out_bytes);
+
+/* dg_attention_dispatch for one block of keys, the way the reference's host loop dispatches
+ * attention_mma_full (enc.rs:2261-2291: blocks in order, blk = {t_begin, t_end, is_first, is_last}
+ * bound at index 7): the first block starts the state in attn_state, a middle block folds its keys
+ * into it, the last block also writes `out`.  A block that is both first and last is
+ * dg_attention_dispatch.  attn_state must hold dg_attention_block_state_bytes() and keep its
+ * contents between the calls of one sequence.  The result equals the single dispatch up to fp32
+ * rounding of the merges (the reference's blocks are bit-identical to its monolithic pass; here
+ * each block is itself split over workgroups, so the sums associate differently). */
+int dg_attention_dispatch_block(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                                const dg_step_params* P, const dg_attn_dims* dims, const dg_attn_block_range* blk,
+                                dg_debug_status* dbg, void* attn_state, size_t attn_state_bytes, void* stream);
+int dg_attention_block_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
+                                   size_t* out_bytes);
 
 /* ---- top-k sparse attention (full-attention layers; the reference's default for them at depth) ----
  *
