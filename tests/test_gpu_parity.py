@@ -154,11 +154,22 @@ def run_workload(po, w, *, n_splits=0, kernel=capi.DG_KERNEL_AUTO, out_f32=False
     return got[rows], got_lse[rows], ref[rows], ref_lse[rows]
 
 
+LSE_ABS = 2.0 ** -8
+
+
 def check_tolerances(got, got_lse, ref, ref_lse, max_abs=MAX_ABS, mean_abs=MEAN_ABS):
+    """The benchmark tolerances on the output; the library's documented bound on the log-sum-exp,
+    |lse - exact| <= max(1e-3 |exact|, 2^-8): the row sum is taken over the probabilities as rounded
+    for the MFMA (the numbers P.V multiplies), which moves ln(sum) by up to 2^-8, so the relative
+    bound alone would fail rows whose LSE is small in magnitude.  Rows without a visible key: -inf."""
     assert np.all(np.isfinite(got))
     assert max_abs_diff(got, ref) <= max_abs
     assert mean_abs_diff(got, ref) <= mean_abs
-    assert np.max(np.abs(got_lse - ref_lse) / np.maximum(np.abs(ref_lse), 1e-6)) <= LSE_REL
+    got_lse, ref_lse = np.asarray(got_lse), np.asarray(ref_lse)
+    ok = np.isfinite(ref_lse)
+    assert np.array_equal(np.isfinite(got_lse), ok)
+    err = np.abs(got_lse[ok] - ref_lse[ok])
+    assert np.all(err <= np.maximum(LSE_REL * np.abs(ref_lse[ok]), LSE_ABS))
 
 
 # ------------------------------------------------------------------ benchmark configurations

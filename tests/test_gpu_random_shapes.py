@@ -6,23 +6,11 @@ import pytest
 
 from diffgemma_amd import attention_topk as T
 from diffgemma_amd import capi, workloads as W
-from test_gpu_parity import MAX_ABS, MEAN_ABS, LSE_REL, run_workload
+from test_gpu_parity import MAX_ABS, MEAN_ABS, check_tolerances, run_workload
 from test_gpu_topk_parity import run_topk
 from helpers import max_abs_diff, mean_abs_diff
 
 pytestmark = pytest.mark.gpu
-
-
-def check_tolerances(got, got_lse, ref, ref_lse):
-    """The benchmark tolerances; for rows whose LSE is small in magnitude the relative bound is
-    replaced by an absolute one: the row sum is taken over probabilities rounded to bf16 (the same
-    numbers P.V multiplies), which moves ln(l) by up to 2^-9."""
-    assert np.all(np.isfinite(got))
-    assert max_abs_diff(got, ref) <= MAX_ABS and mean_abs_diff(got, ref) <= MEAN_ABS
-    ok = np.isfinite(ref_lse)
-    assert np.array_equal(np.isfinite(got_lse), ok)
-    err = np.abs(got_lse[ok] - ref_lse[ok])
-    assert np.all((err <= LSE_REL * np.abs(ref_lse[ok])) | (err <= 2.5e-3))
 
 
 def _case(seed):

@@ -130,6 +130,20 @@ def test_synthetic_fill_kv_range(po):
     assert not np.array_equal(bits, po.synthetic_fill_kv(4096, 12347))
 
 
+def test_synthetic_fill_kv_known_answer(po):
+    """The generator is xorshift64* (shifts 12, 25, 27, multiplier 0x2545F4914F6CDD1D); its published
+    outputs from state 1 are 5180492295206395165, 12380297144915551517, 13389498078930870103.  The fill
+    takes bits 32..47 of an output as r and stores (r & 0x3FF) | 0x3000 | ((r & 0x400) << 5), worked out
+    by hand below: a wrong shift, multiplier, word slice or bit placement changes these words."""
+    #  0x47E4CE4B896CDD1D -> r = 0xCE4B: mantissa 0x24B, bit 10 set   -> 0x8000 | 0x3000 | 0x24B
+    #  0xABCFA6A8E079651D -> r = 0xA6A8: mantissa 0x2A8, bit 10 set   -> 0x8000 | 0x3000 | 0x2A8
+    #  0xB9D10D8FEB731F57 -> r = 0x0D8F: mantissa 0x18F, bit 10 set   -> 0x8000 | 0x3000 | 0x18F
+    want = np.array([0xB24B, 0xB2A8, 0xB18F], dtype=np.uint16)
+    assert np.array_equal(po.synthetic_fill_kv(3, 1), want)
+    assert np.array_equal(po.synthetic_fill_kv(3, 0), want)       # the seed's lowest bit is forced on
+    assert float(want[:1].view(np.float16)[0]) == -(0.125 * (1 + 0x24B / 1024))
+
+
 # ---------------------------------------------------------------- recurrence vs textbook
 @pytest.mark.parametrize("name", list(FIXTURES))
 @pytest.mark.parametrize("strict", [0, 1])
