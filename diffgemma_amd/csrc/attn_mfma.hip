@@ -37,7 +37,7 @@
 // exact as long as nothing overflows.  bf16: tau = 120 with the probabilities stored as
 // 2^(score - reference - 86), so P <= 2^34 and the fp32 sums stay below 2^34 * keys * |v|, far
 // from 2^127; a weight more than 2^40 below the row's running max is stored as an exact zero.
-// With f16 operands P itself has to stay below 65504: tau = 15, no offset.
+// With f16 operands P itself has to stay below 65504: tau = 15.9, no offset.
 #include "attn_params.h"
 #include "mfma_tile.h"
 
@@ -48,7 +48,7 @@ namespace {
 // (a raise rescales a 32-row block of O, which costs about as much as a tile's P.V).  With the
 // offset below the bf16 probabilities then reach 2^34 at most, and a row's sums 2^34 x keys x |v|.
 template <bool F16>
-constexpr float kTau = F16 ? 15.0f : 120.0f;
+constexpr float kTau = F16 ? 15.9f : 120.0f;   // f16: P <= 2^15.9 = 61147, below the largest half (65504)
 // The probabilities are stored as 2^(score - reference - kPOff): with bf16 the offset moves
 // their range to [2^-126, 2^34], so that a key whose weight is below 2^-40 of the reference
 // (and therefore of the row's largest) underflows to an exact zero in the exponential itself.
@@ -415,8 +415,12 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         tmax = max_across_halves(tmax) * p.scale_log2;
         const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kTau<F16>) != 0ull;
         bool rescale = false;   // some row of the block has accumulated something that changes
+        m_run = fmaxf(m_run, tmax);
         if (__builtin_expect(raise, 0)) {
-          const float m_new = fmaxf(m_ref, tmax);
+          // When one row of the block has to raise its reference the whole block is rescaled anyway,
+          // so every row moves its reference up to its running max: the next raise is then as far
+          // away as it can be (with f16 operands, where the threshold is low, this halves the raises).
+          const float m_new = fmaxf(m_ref, m_run);
           const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
           rescale = __builtin_amdgcn_ballot_w64(m_ref != -INFINITY && corr != 1.f) != 0ull;
           l_part *= corr;
@@ -427,10 +431,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         }
         if (lane == 0) ((uint32_t*)(smem + OFF_FLAG + par * FLAG_BYTES))[wave] = rescale ? 1u : 0u;
         m_use = (m_ref == -INFINITY) ? 0.f : m_ref + kPOff<F16>;
-        if constexpr (!F16) {
-          m_run = fmaxf(m_run, tmax);
-          x_drop = m_run - kDrop - m_use;
-        }
+        if constexpr (!F16) x_drop = m_run - kDrop - m_use;
       } else {
         // scores 4 q .. 4 q + 3 in two steps: (a) scale and subtract, first two exponentials;
         // (b) the other two exponentials, rounding to the MFMA operand type, and for every
