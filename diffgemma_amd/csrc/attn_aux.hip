@@ -140,30 +140,33 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
       const bool live = d8_0 + lane < hd / 8;
       const uint32_t d8 = live ? d8_0 + lane : 0u;
       float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      uint32_t s = 0;
-      for (; s + 4 <= p.n_splits; s += 4) {
-        uint4 a[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) a[u] = ((const uint4*)(hbase + (s + u) * sstride))[d8];
+      // Splits whose weight is below 2^-24 of the row's total are left out: what they would add is
+      // under the fp32 rounding of the sum (the weights add up to 1, |O_s| <= the largest |V|), and
+      // on a peaked row, where one split holds nearly all of the mass, most of the partial rows are
+      // then never fetched.  The others are summed in ascending order, four loads in flight.
+      uint64_t todo = __builtin_amdgcn_ballot_w64(lane < p.n_splits && w_half >= 5.9604645e-8f);
+      while (todo != 0ull) {
+        uint32_t idx[4];
+        uint32_t cnt = 0;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const float w = __shfl(w_half, s + u, 64);
+          idx[u] = todo != 0ull ? (uint32_t)__builtin_ctzll(todo) : idx[0];
+          cnt += todo != 0ull ? 1u : 0u;
+          todo &= todo - 1ull;
+        }
+        uint4 a[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a[u] = ((const uint4*)(hbase + idx[u] * sstride))[d8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if ((uint32_t)u >= cnt) break;
+          const float w = __shfl(w_half, (int)idx[u], 64);
           const uint32_t wd[4] = {a[u].x, a[u].y, a[u].z, a[u].w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             acc[2 * e] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] & 0xffffu));
             acc[2 * e + 1] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] >> 16));
           }
-        }
-      }
-      for (; s < p.n_splits; ++s) {
-        const uint4 a = ((const uint4*)(hbase + s * sstride))[d8];
-        const float w = __shfl(w_half, s, 64);
-        const uint32_t wd[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          acc[2 * e] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] & 0xffffu));
-          acc[2 * e + 1] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] >> 16));
         }
       }
       if (!live) continue;
