@@ -538,6 +538,21 @@ def main():
     lse_rel = np.abs(got_lse[toks] - ref_lse[toks]) / np.maximum(np.abs(ref_lse[toks]), 1e-6)
     check = {"rows": int(len(toks)), "max_abs": float(diff.max()), "mean_abs": float(diff.mean()),
              "lse_rel_max": float(lse_rel.max()), "tol": {"max_abs": 2e-2, "mean_abs": 2e-3, "lse_rel": 1e-3}}
+    # How peaked the softmax rows of this data are: the share of (row, key) pairs whose weight is more than
+    # 2^40 below the row's largest.  The bf16 kernel stores those as exact zeros (the matrix cores draw less
+    # power on zero operands, and the kernel's clock is power-limited), so the rate below depends on it.
+    zero_frac = None
+    if w.layout == "head_major" and not w.window:
+        kvr = kv.reshape(2, w.n_kv_heads, w.t_all, w.head_dim)
+        grp = w.n_q_heads // w.n_kv_heads
+        scale = desc.softmax_scale if desc.softmax_scale > 0 else 1.0
+        n_small = n_all = 0
+        for t in toks[:: max(1, len(toks) // 4)]:
+            for h in range(0, w.n_q_heads, max(1, w.n_q_heads // 4)):
+                sc = kvr[0, h // grp] @ q[t, h] * scale
+                n_small += int(np.sum(sc < sc.max() - 40.0 * np.log(2.0)))
+                n_all += sc.size
+        zero_frac = n_small / max(n_all, 1)
     check["passed"] = bool(diff.max() <= 2e-2 and diff.mean() <= 2e-3 and lse_rel.max() <= 1e-3
                            and np.isfinite(got).all())
 
@@ -675,6 +690,7 @@ def main():
         "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "canvas_tokens_per_s": w.canvas / (ms_per_step * 1e-3),
         "flops_per_step": flops, "visible_pairs_per_head": pairs,
+        "softmax_weights_below_2^-40_of_row_max": zero_frac,
         "roofline": {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": kern_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
                      # not read by this run: the counters need the profiler; copied from the committed summary

@@ -80,6 +80,12 @@ def config(name: str) -> Workload:
         return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, sees_masked=True, seed=3)
     if name == "cfg3_global_f16kv":   # config 3 with the reference's storage: bf16 activations, f16 cache
         return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, seed=3, kv_f16=True)
+    if name == "cfg3_global_flat":    # config 3's shape with a flat softmax: scores of unit spread (Q of std 1/sqrt(hd),
+        # no RMSNorm), so that no softmax weight is negligible.  The headline workload's unit-RMS rows without a
+        # 1/sqrt(hd) scale give scores of spread sqrt(hd) and rows so peaked that nearly all weights are stored as
+        # exact zeros, which the power-limited matrix cores reward; this one shows the kernel without that help.
+        return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, rms_norm=False, q_std=1.0 / np.sqrt(512.0),
+                        seed=3)
     if name == "cfg4_long":
         return Workload(name, 256, 16, 2, 512, 131072, rms_norm=False, kv_std=0.5, outlier_frac=0.01,
                         outlier_gain=8.0, seed=4)
