@@ -149,6 +149,46 @@ def test_block_dispatch_equals_single_dispatch(gpu_ready, po, block):
     assert np.abs(g - ref[toks]).max() <= 2e-2 and np.abs(g - ref[toks]).mean() <= 2e-3
 
 
+def test_block_dispatch_replays_in_a_graph(gpu_ready):
+    """The block sequence records no memset node, allocates nothing and synchronises nothing, so it can be
+    captured; replays (with eager work and synchronisations between them) must give the eager bits."""
+    import torch
+    f = A.model_full_fixture(4096 - 256)
+    rig = A.AttnRig.from_fixture(f)
+    lib = capi.load()
+    lo, sp = A.layer_offsets(f), A.step_params(f.kv_len)
+    dims = capi.AttnDims(canvas=f.canvas, n_q_heads=f.n_q_heads, causal=0, window=0)
+    n = C.c_size_t(0)
+    capi.check(lib.dg_attention_block_state_bytes(C.byref(lo), C.byref(dims), f.kv_len, C.byref(n)))
+    st = torch.zeros(n.value, dtype=torch.uint8, device="cuda")
+    t_total, block = f.kv_len + f.canvas, 1500
+    blocks = -(-t_total // block)
+
+    def encode():
+        for b in range(blocks):
+            blk = capi.AttnBlockRange(b * block, min((b + 1) * block, t_total), int(b == 0), int(b + 1 == blocks))
+            capi.check(lib.dg_attention_dispatch_block(rig.buf_q.data_ptr(), rig.buf_kv.data_ptr(), rig.buf_out.data_ptr(),
+                                                       C.byref(lo), C.byref(sp), C.byref(dims), C.byref(blk), None,
+                                                       st.data_ptr(), st.numel(), A.stream_handle()))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        encode()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    want = rig.buf_out.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        encode()
+    for rep in range(3):
+        rig.buf_out.fill_(-1)
+        st.fill_(rep)                 # the carried state of an earlier sequence must not matter
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(rig.buf_out, want), rep
+
+
 def test_partial_argument_checks(gpu_ready):
     import torch
     w = W.scaled(W.config("cfg3_global"), 1024)
