@@ -1,5 +1,6 @@
 // Auxiliary kernels: the scalar cross-check kernel, the split merge, dtype conversion.
 #include "attn_params.h"
+#include "wt_store.h"
 
 #include <hip/hip_fp16.h>
 
@@ -183,7 +184,8 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
         pk.y = (uint32_t)f32_to_bf16_bits(acc[2], tr) | ((uint32_t)f32_to_bf16_bits(acc[3], tr) << 16);
         pk.z = (uint32_t)f32_to_bf16_bits(acc[4], tr) | ((uint32_t)f32_to_bf16_bits(acc[5], tr) << 16);
         pk.w = (uint32_t)f32_to_bf16_bits(acc[6], tr) | ((uint32_t)f32_to_bf16_bits(acc[7], tr) << 16);
-        ((uint4*)((uint16_t*)p.out + ooff))[d8] = pk;
+        const wt_u32x4 pk4 = {pk.x, pk.y, pk.z, pk.w};
+        wt_store16(wt_window_wave((const uint16_t*)p.out + ooff), d8 * 16u, pk4);   // written through: wt_store.h
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) store_out(p, ooff + d8 * 8 + e, acc[e]);
@@ -225,13 +227,15 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
     if (p.dbg && (nonfinite(o.x) || nonfinite(o.y) || nonfinite(o.z) || nonfinite(o.w)))
       dbg_report(p.dbg, 2u, (tok << 16) | qh, d4 * 4u);
     if (p.out_dtype == DT_F32) {
-      ((float4*)((float*)p.out + ooff))[d4] = o;
+      const wt_u32x4 o4 = {__float_as_uint(o.x), __float_as_uint(o.y), __float_as_uint(o.z), __float_as_uint(o.w)};
+      wt_store16(wt_window_wave((const float*)p.out + ooff), d4 * 16u, o4);
     } else if (p.out_dtype == DT_BF16) {   // four bf16 in one 8-byte store
       const bool tr = p.out_trunc != 0;
       uint2 pk;
       pk.x = (uint32_t)f32_to_bf16_bits(o.x, tr) | ((uint32_t)f32_to_bf16_bits(o.y, tr) << 16);
       pk.y = (uint32_t)f32_to_bf16_bits(o.z, tr) | ((uint32_t)f32_to_bf16_bits(o.w, tr) << 16);
-      ((uint2*)((uint16_t*)p.out + ooff))[d4] = pk;
+      const wt_u32x2 pk2 = {pk.x, pk.y};
+      wt_store8(wt_window_wave((const uint16_t*)p.out + ooff), d4 * 8u, pk2);
     } else {
       store_out(p, ooff + d4 * 4 + 0, o.x);
       store_out(p, ooff + d4 * 4 + 1, o.y);

@@ -40,6 +40,7 @@
 // With f16 operands P itself has to stay below 65504: tau = 15.9, no offset.
 #include "attn_params.h"
 #include "mfma_tile.h"
+#include "wt_store.h"
 
 namespace dg {
 namespace {
@@ -637,14 +638,15 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   // row owners publish (m, l) of their rows; d owners normalise and store their slice of O
   const float l_tot = sum_across_halves(l_part + l_part2);
   const float m_pub = m_ref + kPOff<F16>;   // the exponent the sums are relative to
+  // first partial row of this workgroup; partial rows and their (m, l) are written through (wt_store.h)
+  const size_t wg_prow0 = ((size_t)split * p.hkv + kvh) * p.rows_pad + row0;
   __syncthreads();   // the last tile's readers are done with LDS
   if (g2 == 0) {
     sml[(wave * 32u + l32) * 2u] = m_pub;
     sml[(wave * 32u + l32) * 2u + 1u] = l_tot;
     if (p.n_splits > 1) {
-      const size_t prow = ((size_t)split * p.hkv + kvh) * p.rows_pad + r;
-      p.part_ml[prow * 2] = m_pub;
-      p.part_ml[prow * 2 + 1] = l_tot;
+      const u32x2 ml2 = {__float_as_uint(m_pub), __float_as_uint(l_tot)};
+      wt_store8(wt_window(p.part_ml + wg_prow0 * 2), (r - row0) * 8u, ml2);
     } else if (row_ok) {
       if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l_tot > 0.f ? m_pub * kLn2 + __logf(l_tot) : -INFINITY;
       if (p.dbg && !(l_tot > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l_tot));
@@ -676,13 +678,13 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           *(__attribute__((address_space(3))) u32x2*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 2) = h2;
         }
       }
-      const size_t prow0 = ((size_t)split * p.hkv + kvh) * p.rows_pad + row0 + rbk * 32u;
-      uint16_t* const po = (uint16_t*)p.part_o + prow0 * D + 32u * (dgrp * NDBW) + (lane % LPR) * 8u;
+      const auto win = wt_window((const uint16_t*)p.part_o + wg_prow0 * D);
+      const uint32_t po = ((rbk * 32u) * D + 32u * (dgrp * NDBW) + (lane % LPR) * 8u) * 2u;   // bytes
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
         const uint32_t rl = it * RPI + lane / LPR;        // row within the block
         const u32x4 v4 = *(lds_u32x4*)(stg + rl * STG_ROW + (lane % LPR) * 16);
-        *(u32x4*)(po + (size_t)rl * D) = v4;
+        wt_store16(win, po + rl * (D * 2u), v4);
       }
       continue;
     }
@@ -703,13 +705,13 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           *(__attribute__((address_space(3))) f32x4*)(stg + l32 * STG_ROW + (32 * i + 8 * q4 + 4 * g2) * 4) = v4;
         }
       }
-      const size_t prow0 = ((size_t)split * p.hkv + kvh) * p.rows_pad + row0 + rbk * 32u;
-      float* const po = p.part_o + prow0 * D + 32u * (dgrp * NDBW) + (lane % LPR) * 4u;
+      const auto win = wt_window(p.part_o + wg_prow0 * D);
+      const uint32_t po = ((rbk * 32u) * D + 32u * (dgrp * NDBW) + (lane % LPR) * 4u) * 4u;   // bytes
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
         const uint32_t rl = it * RPI + lane / LPR;        // row within the block
-        const f32x4 v4 = *(__attribute__((address_space(3))) f32x4*)(stg + rl * STG_ROW + (lane % LPR) * 16);
-        *(f32x4*)(po + (size_t)rl * D) = v4;
+        const u32x4 v4 = *(lds_u32x4*)(stg + rl * STG_ROW + (lane % LPR) * 16);
+        wt_store16(win, po + rl * (D * 4u), v4);
       }
       continue;
     }
