@@ -9,6 +9,7 @@
 // and V into the cache at slot(pos) in the cache's element type.  HBM-bound by construction:
 // every byte moves once; at 256 canvas rows the launch is a few megabytes, i.e. latency-bound.
 #include "attn_params.h"
+#include "wt_store.h"
 #include "../../include/dg_attn.h"
 
 #include <hip/hip_fp16.h>
@@ -73,18 +74,23 @@ __device__ __forceinline__ void load_row(const uint16_t* src, float (&x)[8]) {
   }
 }
 
-// `per` consecutive elements as 16-bit storage values, packed and written with one store
+// `per` consecutive elements as 16-bit storage values, packed and written with one store at element
+// `d0` of the row that starts at `row` (the same row for the whole wave).  Written through: the
+// attention kernel that follows reads these rows from every XCD (wt_store.h).
 template <int PER>
-__device__ __forceinline__ void store_row16(uint16_t* dst, const uint16_t (&h)[8]) {
+__device__ __forceinline__ void store_row16(uint16_t* row, uint32_t d0, const uint16_t (&h)[8]) {
+  const auto win = wt_window_wave(row);
   if constexpr (PER == 8) {
-    *(uint4*)dst = make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16,
-                              h[6] | (uint32_t)h[7] << 16);
+    const wt_u32x4 v = {h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16,
+                        h[6] | (uint32_t)h[7] << 16};
+    wt_store16(win, d0 * 2u, v);
   } else if constexpr (PER == 4) {
-    *(uint2*)dst = make_uint2(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16);
+    const wt_u32x2 v = {h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16};
+    wt_store8(win, d0 * 2u, v);
   } else if constexpr (PER == 2) {
-    *(uint32_t*)dst = h[0] | (uint32_t)h[1] << 16;
+    wt_store4(win, d0 * 2u, h[0] | (uint32_t)h[1] << 16);
   } else {
-    dst[0] = h[0];
+    wt_store2(win, d0 * 2u, h[0]);
   }
 }
 
@@ -129,7 +135,7 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
     if (kv_write && active) {
 #pragma unroll
       for (int i = 0; i < PER; ++i) bits[i] = cache_bits(p.kv_dtype, x[i] * inv);
-      store_row16<PER>((uint16_t*)p.vc + slot * p.v_tok_stride + (int64_t)hh * p.v_head_stride + d0, bits);
+      store_row16<PER>((uint16_t*)p.vc + slot * p.v_tok_stride + (int64_t)hh * p.v_head_stride, d0, bits);
     }
     return;
   }
@@ -162,13 +168,13 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   if (is_k && kv_write) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) bits[i] = cache_bits(p.kv_dtype, y[i]);
-    store_row16<PER>((uint16_t*)p.kc + slot * p.k_tok_stride + (int64_t)hh * p.k_head_stride + d0, bits);
+    store_row16<PER>((uint16_t*)p.kc + slot * p.k_tok_stride + (int64_t)hh * p.k_head_stride, d0, bits);
   }
   // Q always goes back in place; K only when V does not alias the raw k projection (cpu.rs:137-143)
   if (is_q || !p.v_from_k) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) bits[i] = f32_to_bf16_bits(y[i], p.qk_trunc != 0);
-    store_row16<PER>(row_inplace + d0, bits);
+    store_row16<PER>(row_inplace, d0, bits);
   }
 }
 

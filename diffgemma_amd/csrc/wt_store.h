@@ -46,5 +46,9 @@ __device__ __forceinline__ void wt_store4(__amdgpu_buffer_rsrc_t w, uint32_t byt
   __builtin_amdgcn_raw_buffer_store_b32(v, w, byte_off, 0, kWtPolicy);
 }
 
+__device__ __forceinline__ void wt_store2(__amdgpu_buffer_rsrc_t w, uint32_t byte_off, uint16_t v) {
+  __builtin_amdgcn_raw_buffer_store_b16(v, w, byte_off, 0, kWtPolicy);
+}
+
 }  // namespace
 }  // namespace dg
