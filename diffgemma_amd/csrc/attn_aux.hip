@@ -249,6 +249,85 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
   }
 }
 
+// The same merge for at most 8 splits of f16 partial rows whose total is small (a sliding layer:
+// 6 splits x 4096 rows x 512 bytes): there the kernel is as long as one wave's chain of memory round
+// trips, not bandwidth.  So a wave asks for everything at once, the (m, l) pairs and the partial rows
+// of all splits (an absent split repeats the last one, weight zero), instead of weights first and
+// only the rows of splits that count; and the weights come from lane-to-scalar reads, every lane
+// doing the same arithmetic, instead of a dozen dependent shuffles.  The sum of the weights pairs
+// its terms as the butterfly over the lanes does, ((0+4)+(2+6))+((1+5)+(3+7)), and the rows are
+// added in the same order with the same cut, so both kernels give the same bits.
+constexpr uint32_t kMergeFewSplits = 8;
+__global__ void __launch_bounds__(256) attn_merge_few_kernel(const AttnParams p, const uint32_t hd) {
+  const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t gr = blockIdx.x * 4 + wave;  // global stacked row over all KV heads
+  if (gr >= p.hkv * p.rows_total) return;
+  const uint32_t kvh = gr / p.rows_total, r = gr % p.rows_total;
+  const uint32_t tok = r / p.group, qh = kvh * p.group + r % p.group;
+  const size_t split_stride = (size_t)p.hkv * p.rows_pad;
+  const size_t row = (size_t)kvh * p.rows_pad + r;
+  const uint32_t n = p.n_splits;
+  const float2 ml = *(const float2*)(p.part_ml + ((size_t)min(lane, n - 1u) * split_stride + row) * 2);
+  const bool live = lane < hd / 8;
+  const uint32_t d8 = live ? lane : 0u;
+  const uint16_t* const hbase = (const uint16_t*)p.part_o + row * hd;
+  const size_t sstride = split_stride * hd;
+  uint4 a[kMergeFewSplits];
+#pragma unroll
+  for (uint32_t u = 0; u < kMergeFewSplits; ++u) a[u] = ((const uint4*)(hbase + min(u, n - 1u) * sstride))[d8];
+  float msu[kMergeFewSplits], wlu[kMergeFewSplits];
+  float mx = -INFINITY;
+#pragma unroll
+  for (uint32_t u = 0; u < kMergeFewSplits; ++u) {
+    msu[u] = u < n ? __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(ml.x), (int)u)) : -INFINITY;
+    mx = fmaxf(mx, msu[u]);
+  }
+#pragma unroll
+  for (uint32_t u = 0; u < kMergeFewSplits; ++u) {
+    const float lsu = u < n ? __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(ml.y), (int)u)) : 0.f;
+    wlu[u] = lsu > 0.f ? lsu * exp2f(msu[u] - mx) : 0.f;
+  }
+  const float den = ((wlu[0] + wlu[4]) + (wlu[2] + wlu[6])) + ((wlu[1] + wlu[5]) + (wlu[3] + wlu[7]));
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (uint32_t u = 0; u < kMergeFewSplits; ++u) {
+    const float w = wlu[u] * inv;
+    if (u < n && w >= 5.9604645e-8f) {   // the same in every lane
+      const uint32_t wd[4] = {a[u].x, a[u].y, a[u].z, a[u].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] & 0xffffu));
+        acc[2 * e + 1] += w * (float)__builtin_bit_cast(_Float16, (uint16_t)(wd[e] >> 16));
+      }
+    }
+  }
+  const size_t ooff = ((size_t)tok * p.hq + qh) * hd;
+  if (live) {
+    if (p.dbg) {
+      bool bad = false;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bad = bad || nonfinite(acc[e]);
+      if (bad) dbg_report(p.dbg, 2u, (tok << 16) | qh, d8 * 8u);
+    }
+    if (p.out_dtype == DT_BF16) {
+      const bool tr = p.out_trunc != 0;
+      const wt_u32x4 pk4 = {(uint32_t)f32_to_bf16_bits(acc[0], tr) | ((uint32_t)f32_to_bf16_bits(acc[1], tr) << 16),
+                            (uint32_t)f32_to_bf16_bits(acc[2], tr) | ((uint32_t)f32_to_bf16_bits(acc[3], tr) << 16),
+                            (uint32_t)f32_to_bf16_bits(acc[4], tr) | ((uint32_t)f32_to_bf16_bits(acc[5], tr) << 16),
+                            (uint32_t)f32_to_bf16_bits(acc[6], tr) | ((uint32_t)f32_to_bf16_bits(acc[7], tr) << 16)};
+      wt_store16(wt_window_wave((const uint16_t*)p.out + ooff), d8 * 16u, pk4);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) store_out(p, ooff + d8 * 8 + e, acc[e]);
+    }
+  }
+  if (lane == 0) {
+    if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));
+    if (p.lse) p.lse[(size_t)tok * p.hq + qh] = den > 0.f ? mx * kLn2 + logf(den) : -INFINITY;
+  }
+}
+
 __device__ __forceinline__ float load_any(const void* src, uint32_t dt, size_t i) {
   if (dt == DT_F32) return ((const float*)src)[i];
   if (dt == DT_BF16) return bf16_bits_to_f32(((const uint16_t*)src)[i]);
@@ -469,9 +548,14 @@ hipError_t launch_state_merge(const StateMergeParams& p, hipStream_t s) {
   return hipGetLastError();
 }
 
-hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, hipStream_t s) {
+hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, bool streamed, hipStream_t s) {
   const uint32_t rows = p.hkv * p.rows_total;
-  hipLaunchKernelGGL(attn_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, p, head_dim);
+  // a few splits of a small workspace: the variant that asks for every partial row up front
+  const size_t part_bytes = (size_t)p.n_splits * p.hkv * p.rows_pad * head_dim * 2;
+  if (!streamed && p.part_half && p.n_splits <= kMergeFewSplits && head_dim % 8 == 0 && head_dim <= 512 && part_bytes <= ((size_t)32 << 20))
+    hipLaunchKernelGGL(attn_merge_few_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, p, head_dim);
+  else
+    hipLaunchKernelGGL(attn_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, p, head_dim);
   return hipGetLastError();
 }
 

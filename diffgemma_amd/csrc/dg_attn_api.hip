@@ -189,12 +189,13 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl, const uint32_t* key_rang
   if (pl->scalar) {
     splits = 1;
   } else if (splits == 0) {
-    // enough workgroups for every CU, but no split shorter than 8 tiles: below that the partial
+    // enough workgroups for every CU, but no split shorter than 6 tiles: below that the partial
     // rows a split writes (and the merge reads back) cost more than the idle CUs do (a sliding
-    // layer's 40 tiles: 5 splits 25.6-26.3 us, 8 splits 27.4, 4 splits 26.3, 3 splits 29.1)
+    // layer's 40 tiles, step in us: 4 splits 25.7, 5 splits 24.8, 6 and 7 splits 23.7, 8 splits 24.5,
+    // 10 splits 33.4)
     const uint32_t base = d->n_kv_heads * pl->n_mtiles;
     splits = std::max(1u, (uint32_t)cus / std::max(1u, base));
-    splits = std::min(splits, std::max(1u, ntiles / 8u));
+    splits = std::min(splits, std::max(1u, ntiles / 6u));
   }
   splits = std::min(std::min(splits, kMaxSplits), ntiles);
   pl->tiles_per_split = (ntiles + splits - 1) / splits;
@@ -414,7 +415,7 @@ int forward_planned(const dg_attn_desc* d, const Plan& pl, const void* q, const 
     (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 1], s);
     ++g_prof.used;
   }
-  if (pl.n_splits > 1 && dg::launch_attn_merge(p, hd, s) != hipSuccess) return DG_ERR_LAUNCH;
+  if (pl.n_splits > 1 && dg::launch_attn_merge(p, hd, (d->flags & DG_ATTN_F_STREAMED_MERGE) != 0, s) != hipSuccess) return DG_ERR_LAUNCH;
   return DG_OK;
 }
 }  // namespace

@@ -86,6 +86,10 @@ def config(name: str) -> Workload:
         # exact zeros, which the power-limited matrix cores reward; this one shows the kernel without that help.
         return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, rms_norm=False, q_std=1.0 / np.sqrt(512.0),
                         seed=3)
+    if name == "cfg3_global_flat_f16kv":   # the flat-softmax variant over an f16 cache: no row's maximum moves far
+        # enough to outrun f16 probabilities, so the f16 kernel shows without its rescales of O
+        return Workload(name, 256, 16, 2, 512, 32768, causal_rows=128, rms_norm=False, q_std=1.0 / np.sqrt(512.0),
+                        seed=3, kv_f16=True)
     if name == "cfg4_long":
         return Workload(name, 256, 16, 2, 512, 131072, rms_norm=False, kv_std=0.5, outlier_frac=0.01,
                         outlier_gain=8.0, seed=4)

@@ -74,6 +74,11 @@ typedef enum dg_kernel_sel {
                                               the range saturate.  This is the default for an f16
                                               cache, which guarantees the range; the rounding is 1/8 of
                                               a bf16 output's. */
+#define DG_ATTN_F_STREAMED_MERGE 0x20u     /* merge the split partial rows with the streaming kernel (weights
+                                              first, then only the rows of splits that count) even where the
+                                              library would pick the one that fetches every partial row up
+                                              front (at most 8 splits, f16 partial rows, workspace up to
+                                              32 MiB).  Both give the same bits; the flag is there to compare them. */
 
 typedef struct dg_attn_desc {
   uint32_t canvas;        /* query rows; the reference passes active_canvas (256/128/64) */

@@ -253,6 +253,32 @@ def test_split_partial_formats(gpu_ready, po, hd, hq, hkv, splits):
     assert np.array_equal(f32a[0], f32b[0])
 
 
+@pytest.mark.parametrize("hd,hq,hkv,splits,canvas", [(256, 16, 8, 6, 256), (256, 16, 8, 8, 100), (512, 16, 2, 8, 64),
+                                                     (128, 8, 4, 3, 77), (64, 8, 8, 2, 33), (32, 4, 4, 5, 20)])
+def test_both_merge_kernels_give_the_same_bits(gpu_ready, hd, hq, hkv, splits, canvas):
+    """A few splits over a small workspace are merged by the kernel that fetches every partial row up front;
+    DG_ATTN_F_STREAMED_MERGE asks for the streaming one instead.  Same weights, same cut of negligible
+    splits, same order of the sums: output and LSE are bit-equal (peaked rows, so that the cut is taken)."""
+    import torch
+    w = W.Workload("merge_ab", canvas, hq, hkv, hd, 2049, causal_rows=canvas // 2, seed=13)
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+
+    def run(flags):     # bf16 output, f16 partial rows (the workload descriptor asks for them)
+        desc = w.desc(n_splits=splits, flags=flags)
+        out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.int16, device="cuda")
+        lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+        A.forward(desc, qd, kd, out, lse, A.alloc_workspace(desc))
+        torch.cuda.synchronize()
+        return out.cpu().numpy().view(np.uint16), lse.cpu().numpy()
+
+    a, a_lse = run(0)
+    b, b_lse = run(capi.DG_ATTN_F_STREAMED_MERGE)
+    assert np.array_equal(a, b)
+    assert np.array_equal(a_lse.view(np.uint32), b_lse.view(np.uint32))
+    assert np.isfinite(a_lse).all() and np.any(a != 0)
+
+
 def test_dropped_weights_stay_below_rounding(gpu_ready, po):
     """The kernel stores a softmax weight that is more than 2^40 below its row's running max as an exact
     zero.  Rows built to make the most of that: one key at the top, half of the others 2^39 below it (kept),
