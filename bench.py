@@ -35,6 +35,8 @@ def parse_args():
     ap.add_argument("--global-topk", action="store_true",
                     help="cfg5_schedule: run the global layers as top-k sparse attention (the reference's default for them)")
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--streamed-merge", action="store_true",
+                    help="merge split partial rows with the streaming kernel even where the up-front one would be picked")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline sample time")
     ap.add_argument("--check-toks", type=int, default=12)
@@ -510,7 +512,7 @@ def main():
     q, kv = W.generate(w)
     qd, kd = W.device_arrays(w, q, kv)
     t_gen = time.perf_counter() - t_gen
-    desc = w.desc(n_splits=args.splits)
+    desc = w.desc(n_splits=args.splits, flags=capi.DG_ATTN_F_STREAMED_MERGE if args.streamed_merge else 0)
     pairs, flops = capi.visible_pairs(desc)
     n_splits = capi.resolved_splits(desc)
     out_dt = torch.int16 if w.dtype == "bf16" else torch.float32

@@ -552,7 +552,7 @@ hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, bool stream
   const uint32_t rows = p.hkv * p.rows_total;
   // a few splits of a small workspace: the variant that asks for every partial row up front
   const size_t part_bytes = (size_t)p.n_splits * p.hkv * p.rows_pad * head_dim * 2;
-  if (!streamed && p.part_half && p.n_splits <= kMergeFewSplits && head_dim % 8 == 0 && head_dim <= 512 && part_bytes <= ((size_t)32 << 20))
+  if (!streamed && p.part_half && p.n_splits <= kMergeFewSplits && head_dim % 8 == 0 && head_dim <= 512 && part_bytes < ((size_t)32 << 20))
     hipLaunchKernelGGL(attn_merge_few_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, p, head_dim);
   else
     hipLaunchKernelGGL(attn_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, p, head_dim);

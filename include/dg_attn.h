@@ -77,7 +77,7 @@ typedef enum dg_kernel_sel {
 #define DG_ATTN_F_STREAMED_MERGE 0x20u     /* merge the split partial rows with the streaming kernel (weights
                                               first, then only the rows of splits that count) even where the
                                               library would pick the one that fetches every partial row up
-                                              front (at most 8 splits, f16 partial rows, workspace up to
+                                              front (at most 8 splits, f16 partial rows, workspace below
                                               32 MiB).  Both give the same bits; the flag is there to compare them. */
 
 typedef struct dg_attn_desc {
