@@ -16,6 +16,7 @@ DG_ATTN_F_T_LO_EXPLICIT = 0x4
 DG_ATTN_F_F32_PARTIALS = 0x8
 DG_ATTN_F_F16_PARTIALS = 0x10
 DG_ATTN_F_STREAMED_MERGE = 0x20
+DG_ATTN_F_KV_FROM_HBM = 0x40
 DG_DBG_ATTN_NONPOSITIVE_L = 1
 DG_DBG_ATTN_NONFINITE_OUT = 2
 DG_DBG_KERNEL_ATTENTION = 7

@@ -158,7 +158,7 @@ __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
   }
 }
 
-template <int D, bool F16>
+template <int D, bool F16, bool TOUCH>
 __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   using L = Lay<D>;
   constexpr int NSTEP = D / 16, NDB = D / 32;
@@ -176,7 +176,22 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   constexpr int P_BYTES = 2 * 4 * 1024, CORR_BYTES = 4 * 32 * 4, FLAG_BYTES = 16;
   constexpr int OFF_P = 2 * L::K_BYTES + 2 * L::V_BYTES, OFF_CORR = OFF_P + 2 * P_BYTES;
   constexpr int OFF_FLAG = OFF_CORR + 2 * CORR_BYTES, OFF_ML = OFF_FLAG + 2 * FLAG_BYTES;
-  constexpr int LDS_BYTES = OFF_ML + 4 * 32 * 2 * 4;
+  // At head_dim 512, when the caller says the cache rows will come from HBM (AttnParams.touch_ahead,
+  // which selects the TOUCH instance of the kernel: the other one has none of this in its loop),
+  // the key and value tiles a workgroup will need are touched into the L2 PF_AHEAD tiles before their
+  // loads to LDS are issued (with the rows in the memory-side cache after all the touches cost 2 %:
+  // they sit in the same in-order queue as the tile loads).  Two tile buffers per matrix and one barrier per tile
+  // leave a load one tile's time (1.7 us) to land, less for the loads issued late in the tile; that
+  // covers the memory-side cache and not HBM under load: with the cache of a 32k-key layer not
+  // resident (a schedule of 30 layers streams 1.1 GB per iteration) the workgroups took 14 % more
+  // cycles at an unchanged clock.  The touch is the most recent load at every barrier of the tile
+  // loop, which waits for all loads but that one, so a touch has until the barrier after the next.
+  constexpr bool PREFETCH = TOUCH;
+  static_assert(!TOUCH || D == 512, "a row of 1 KiB = 8 lines is assumed");
+  constexpr int PF_AHEAD = 6;
+  constexpr int OFF_DUMP = OFF_ML + 4 * 32 * 2 * 4;
+  constexpr int LDS_BYTES = OFF_DUMP + (PREFETCH ? 256 : 0);
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS of one compute unit");
   static_assert(L::K_BYTES % 16 == 0 && L::V_BYTES % 16 == 0, "buffer alignment");
   __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
   float* const sml = (float*)(smem + OFF_ML);
@@ -251,6 +266,38 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const uint32_t te = __builtin_amdgcn_readfirstlane(min(tb + per_split, mt_end));
   const uint32_t ntile = te > tb ? te - tb : 0u;
 
+  const char* kbase = (const char*)p.k + (int64_t)kvh * p.k_head_stride * 2;
+  const char* vbase = (const char*)p.v + (int64_t)kvh * p.v_head_stride * 2;
+  const int64_t kstride_b = p.k_tok_stride * 2, vstride_b = p.v_tok_stride * 2;
+  // Touch this workgroup's share of key tile `tile` of the split (the last tile instead of one past it).
+  // The row tiles of a (KV head, split) pair stream the same keys behind one L2, so they share the
+  // work: a tile is 256 lines of K and 256 of V (a row is 1 KiB = 8 lines), row tile mt takes the
+  // eighth (mt mod 8) of them, 16 lines per wave in one instruction (the other lanes repeat them).
+  // Every workgroup touching whole tiles cost more in the load pipeline than the misses it saved.
+  struct Touch {
+    const char* base;   // wave-uniform
+    uint32_t voff;      // per lane
+  };
+  auto touch_address = [&](uint32_t tile, uint32_t ln) -> Touch {
+    const uint32_t tp = min(tile, te - 1u) * kBlockN;
+    const uint32_t share = mt & 7u;
+    const bool is_v = share >= 4u;
+    const uint32_t li = (share & 3u) * 64u + wave * 16u + (ln & 15u);
+    const uint32_t row = min(li >> 3, p.t_all - 1u - tp);
+    const int64_t stride_b = is_v ? vstride_b : kstride_b;
+    const int64_t slot = (int64_t)kv_slot(p.ring_mask, tp);
+    return Touch{(is_v ? vbase : kbase) + slot * stride_b, row * (uint32_t)stride_b + (li & 7u) * 128u};
+  };
+  auto touch = [&](const Touch& t) { lds_dma_touch(t.base, t.voff, (uint32_t)(size_t)(smem + OFF_DUMP)); };
+  auto touch_tile = [&](uint32_t tile, uint32_t ln) { touch(touch_address(tile, ln)); };
+  if constexpr (PREFETCH) {
+    // tiles 0 .. 2 are loaded right away; 3 .. PF_AHEAD - 2 are touched here (the wait for the query rows
+    // covers them), PF_AHEAD - 1 before the loop and PF_AHEAD + jj during tile jj
+    if (ntile > 3) {
+      static_for<3, PF_AHEAD - 1>([&](auto i_c) { touch_tile(tb + decltype(i_c)::value, lane); });
+    }
+  }
+
   // ---- Q fragments: B operand of S^T = K.Q^T, lane = row, 8 consecutive d per step ----
   // The operand layout gives a lane 16 bytes of its own row per step, so loading the fragments
   // straight from memory touches 32 bytes of 32 different cache lines per instruction, and the
@@ -316,10 +363,6 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   float x_drop = -INFINITY; // exponents below this are dropped: m_run - kDrop, relative to the reference in use
   float l_part = 0.f;       // this lane's share of the row sum (its 16 of every 32 keys),
   float l_part2 = 0.f;      // kept as two partial sums
-
-  const char* kbase = (const char*)p.k + (int64_t)kvh * p.k_head_stride * 2;
-  const char* vbase = (const char*)p.v + (int64_t)kvh * p.v_head_stride * 2;
-  const int64_t kstride_b = p.k_tok_stride * 2, vstride_b = p.v_tok_stride * 2;
 
   // per-lane LDS byte offsets of the fragment reads (everything else is a compile-time offset
   // in the padded layout, or one XOR with a per-lane constant in the swizzled one)
@@ -519,6 +562,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
     qk_steps(I0{}, IQK{}, k0, std::false_type{}, std::true_type{}, s_a, s_b, 0u, 0u, nothing);
     __syncthreads();   // every wave is done with K(tb): its buffer takes K(tb+2)
     issue_tile<D, false>(k_load((tb + 2) * kBlockN, k0, lane), wave, lane);
+    if constexpr (PREFETCH) touch_tile(tb + PF_AHEAD - 1, lane);
     kf_preload(k1);
 
     for (uint32_t jj = 0; jj < ntile; ++jj) {
@@ -542,7 +586,8 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // the rescale words and V(jj) of this tile are visible to the d owners; every wave is done
       // reading K(jj+1), V(jj-1) and the previous tile's P (which has its own buffer), so their
       // buffers can be refilled.
-      wait_vmem_all();
+      if constexpr (PREFETCH) wait_vmem_but<1>();   // (the touch of the previous tile may be on its way)
+      else wait_vmem_all();
       __syncthreads();
 
       // ---- d-owner role ----
@@ -567,6 +612,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       // than this kernel has.
       const uint32_t lane_l = opaque(lane);
       TileLoad next_v, next_k;
+      Touch next_touch{nullptr, 0u};
       qk_steps(ISPLIT{}, IQK{}, kb_next, std::true_type{}, std::false_type{}, s_b, s_a, t0, par, [&](auto st_c) {
         constexpr int st = decltype(st_c)::value;
         if constexpr (st == NSPLIT) next_v = pinned(v_load(t0 + kBlockN, vb_free, lane_l));
@@ -623,6 +669,20 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
           }
           if constexpr (NPV >= 16 && n >= COPY_AT && n < COPY_AT + 8) copy_scores_part<n - COPY_AT>(s_a, s_b);
           if constexpr (NPV >= PFK && n >= NPV - PFK) kf[n - (NPV - PFK)] = k_frag(kb_next2, n - (NPV - PFK));
+          // the touch itself behind the tile's last load, its address worked out a few MFMAs earlier
+          // (behind the last MFMA nothing would overlap the arithmetic)
+          if constexpr (PREFETCH && n == NPV - 6) {
+            next_touch = touch_address(tb + jj + PF_AHEAD, lane_l);
+            uint64_t b = (uint64_t)next_touch.base;
+            uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+            uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+            asm volatile("" : "+s"(lo), "+s"(hi), "+v"(next_touch.voff));
+            next_touch.base = (const char*)(((uint64_t)hi << 32) | lo);
+          }
+          if constexpr (PREFETCH && n == NPV - 1) {
+            static_assert(!PREFETCH || (2 * NLD - 1) * LD_EVERY < NPV - 1, "the touch follows the tile's last load");
+            touch(next_touch);
+          }
         });
         if constexpr (f + PFV + 1 < NVF) va[f % (PFV + 1)] = v_frag_n(f + PFV + 1);
       });
@@ -754,7 +814,13 @@ template <int D, bool F16>
 hipError_t launch_one(const AttnParams& p, hipStream_t s) {
   const uint32_t nstream = p.hkv * p.n_splits;
   const uint32_t grid = ((nstream * p.n_mtiles + 7u) / 8u) * 8u;
-  hipLaunchKernelGGL((attn_mfma_kernel<D, F16>), dim3(grid), dim3(256), 0, s, p);
+  if constexpr (D == 512) {
+    if (p.touch_ahead) {
+      hipLaunchKernelGGL((attn_mfma_kernel<D, F16, true>), dim3(grid), dim3(256), 0, s, p);
+      return hipGetLastError();
+    }
+  }
+  hipLaunchKernelGGL((attn_mfma_kernel<D, F16, false>), dim3(grid), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 

@@ -40,6 +40,7 @@ struct AttnParams {
   uint32_t q_is_bf16;    // Q holds bf16 although E is f16 (reference: bf16 activations, f16 cache)
   uint32_t out_dtype, out_trunc;
   uint32_t part_half;    // split partials are normalised f16 rows instead of unnormalised fp32 ones
+  uint32_t touch_ahead;  // head_dim 512: touch key/value tiles into the L2 some tiles before they are loaded
   float scale_log2;      // softmax_scale * log2(e)
 };
 

@@ -377,6 +377,7 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   p.out_dtype = d->out_dtype;
   p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
   p.part_half = pl.part_half ? 1u : 0u;
+  p.touch_ahead = (d->flags & DG_ATTN_F_KV_FROM_HBM) ? 1u : 0u;
   p.scale_log2 = pl.scale * dg::kLog2e;
   return DG_OK;
 }

@@ -75,6 +75,14 @@ __device__ __forceinline__ void wait_vmem_all() {
   asm volatile("" ::: "memory");
 }
 
+// all but the N most recent vector memory operations of the wave (they complete in order)
+template <int N>
+__device__ __forceinline__ void wait_vmem_but() {
+  static_assert(N >= 0 && N < 16, "low four bits of vmcnt");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+  asm volatile("" ::: "memory");
+}
+
 // value of lane l combined with lane l^32
 __device__ __forceinline__ float max_across_halves(float x) {
   const uint32_t u = __float_as_uint(x);
@@ -195,6 +203,15 @@ __device__ __forceinline__ void lds_dma_16(const char* base_uniform, uint32_t vo
                  "s"(base), "n"(LDS_IMM)
                  : "memory", "scc");
   }
+}
+
+// lane l: 4 bytes from base + voff -> a dump area in LDS (64 words) that nobody reads.  What the load
+// is for is its side effect: the 128-byte line it touches is in the L2 afterwards.  A load without a
+// register destination, so nothing has to stay reserved until it lands.
+__device__ __forceinline__ void lds_dma_touch(const char* base_uniform, uint32_t voff, uint32_t lds_dump_uniform) {
+  const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_dump_uniform);
+  const uint64_t base = uniform_address(base_uniform);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(voff), "s"(base) : "memory");
 }
 
 template <int D, bool IS_V, int K>

@@ -74,6 +74,13 @@ typedef enum dg_kernel_sel {
                                               the range saturate.  This is the default for an f16
                                               cache, which guarantees the range; the rounding is 1/8 of
                                               a bf16 output's. */
+#define DG_ATTN_F_KV_FROM_HBM 0x40u        /* hint: the cache rows this call reads will not be in the
+                                              memory-side cache (256 MB on MI355X) when it runs, as in a loop
+                                              over many layers whose caches add up to more than that.  The
+                                              head_dim 512 kernel then touches key/value tiles into the L2
+                                              six tiles before it loads them: 5 % faster when the rows do come
+                                              from HBM, 2 % slower when they were cached after all.  Results
+                                              are the same bits either way. */
 #define DG_ATTN_F_STREAMED_MERGE 0x20u     /* merge the split partial rows with the streaming kernel (weights
                                               first, then only the rows of splits that count) even where the
                                               library would pick the one that fetches every partial row up

@@ -279,6 +279,31 @@ def test_both_merge_kernels_give_the_same_bits(gpu_ready, hd, hq, hkv, splits, c
     assert np.isfinite(a_lse).all() and np.any(a != 0)
 
 
+@pytest.mark.parametrize("canvas,hq,hkv,kv_len,splits", [(256, 16, 2, 32768, 0), (64, 16, 2, 1000, 0), (100, 8, 1, 2049, 3),
+                                                         (33, 8, 2, 70, 1), (256, 16, 2, 4099, 8)])
+def test_kv_from_hbm_hint_changes_no_bit(gpu_ready, canvas, hq, hkv, kv_len, splits):
+    """DG_ATTN_F_KV_FROM_HBM selects the head_dim 512 kernel that touches key/value tiles into the L2 ahead
+    of their loads: a change in timing only.  Ragged last tiles, splits shorter than the look-ahead and a
+    single tile included."""
+    import torch
+    w = W.Workload("hint", canvas, hq, hkv, 512, kv_len, causal_rows=canvas // 2, seed=17)
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+
+    def run(flags):
+        desc = w.desc(n_splits=splits, flags=flags)
+        out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.int16, device="cuda")
+        lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+        A.forward(desc, qd, kd, out, lse, A.alloc_workspace(desc))
+        torch.cuda.synchronize()
+        return out.cpu().numpy().view(np.uint16), lse.cpu().numpy()
+
+    a, a_lse = run(0)
+    b, b_lse = run(capi.DG_ATTN_F_KV_FROM_HBM)
+    assert np.array_equal(a, b) and np.array_equal(a_lse.view(np.uint32), b_lse.view(np.uint32))
+    assert np.isfinite(a_lse).all() and np.any(a != 0)
+
+
 def test_dropped_weights_stay_below_rounding(gpu_ready, po):
     """The kernel stores a softmax weight that is more than 2^40 below its row's running max as an exact
     zero.  Rows built to make the most of that: one key at the top, half of the others 2^39 below it (kept),
