@@ -102,8 +102,8 @@ def test_layout_helpers():
 def test_split_planning():
     assert capi.resolved_splits(W.config("cfg3_global").desc()) == 8          # 32 (tile, head) pairs x 8 = 256 workgroups
     assert capi.resolved_splits(W.config("cfg4_long").desc()) == 8
-    assert capi.resolved_splits(W.config("cfg2_sliding").desc()) == 5            # 40 visible tiles, none shorter than 8
-    assert capi.resolved_splits(W.config("cfg2_sliding_768").desc()) == 4        # 32 visible tiles
+    assert capi.resolved_splits(W.config("cfg2_sliding").desc()) == 6            # 40 visible tiles, 7 to a split (none shorter than 6)
+    assert capi.resolved_splits(W.config("cfg2_sliding_768").desc()) == 5        # 32 visible tiles, 7 to a split
     assert capi.resolved_splits(A.make_desc(2, 4, 2, 32, 2)) == 1                 # one tile: nothing to split
     assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, n_splits=3)) == 3
     assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, kernel=capi.DG_KERNEL_SCALAR)) == 1
