@@ -271,18 +271,20 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
   const int64_t kstride_b = p.k_tok_stride * 2, vstride_b = p.v_tok_stride * 2;
   // Touch this workgroup's share of key tile `tile` of the split (the last tile instead of one past it).
   // The row tiles of a (KV head, split) pair stream the same keys behind one L2, so they share the
-  // work: a tile is 256 lines of K and 256 of V (a row is 1 KiB = 8 lines), row tile mt takes the
-  // eighth (mt mod 8) of them, 16 lines per wave in one instruction (the other lanes repeat them).
-  // Every workgroup touching whole tiles cost more in the load pipeline than the misses it saved.
+  // work: a tile is 256 lines of K and 256 of V (a row is 1 KiB = 8 lines); with 16 row tiles or more,
+  // row tile mt takes the sixteenth (mt mod 16) of them, 8 lines per wave in one instruction (the
+  // other lanes repeat them); with fewer, an eighth.  Every workgroup touching whole tiles cost more
+  // in the load pipeline than the misses it saved.
   struct Touch {
     const char* base;   // wave-uniform
     uint32_t voff;      // per lane
   };
   auto touch_address = [&](uint32_t tile, uint32_t ln) -> Touch {
     const uint32_t tp = min(tile, te - 1u) * kBlockN;
-    const uint32_t share = mt & 7u;
-    const bool is_v = share >= 4u;
-    const uint32_t li = (share & 3u) * 64u + wave * 16u + (ln & 15u);
+    const uint32_t sh = p.n_mtiles >= 16u ? 4u : 3u;   // log2 of the number of shares
+    const uint32_t share = mt & ((1u << sh) - 1u);
+    const bool is_v = (share >> (sh - 1u)) != 0u;      // the upper half of the shares are V's lines
+    const uint32_t li = (share & ((1u << (sh - 1u)) - 1u)) * (512u >> sh) + wave * (128u >> sh) + (ln & ((128u >> sh) - 1u));
     const uint32_t row = min(li >> 3, p.t_all - 1u - tp);
     const int64_t stride_b = is_v ? vstride_b : kstride_b;
     const int64_t slot = (int64_t)kv_slot(p.ring_mask, tp);
