@@ -80,7 +80,8 @@ typedef enum dg_kernel_sel {
                                               head_dim 512 kernel then touches key/value tiles into the L2
                                               six tiles before it loads them: 5 % faster when the rows do come
                                               from HBM, 2 % slower when they were cached after all.  Results
-                                              are the same bits either way. */
+                                              are the same bits either way.  A call that streams more than
+                                              256 MiB of keys and values does this without being told. */
 #define DG_ATTN_F_STREAMED_MERGE 0x20u     /* merge the split partial rows with the streaming kernel (weights
                                               first, then only the rows of splits that count) even where the
                                               library would pick the one that fetches every partial row up
