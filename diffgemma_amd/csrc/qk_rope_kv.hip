@@ -5,7 +5,7 @@
 // One wave per (canvas row, head), heads = Hq query heads, then Hkv key heads, then Hkv value
 // heads, exactly the reference's grid (enc.rs:1794-1804).  The row (at most 1 KiB) is read once
 // with up to 16-byte loads, normalised in registers, staged in LDS where each lane rotates one
-// pair (d, hd/2 + d) per pass (one sincos per pair), and written once: Q (and K, unless V aliases it) back in place as bf16, K
+// pair (d, hd/2 + d) per pass (cos and sin of the row's angles once per workgroup of four heads), and written once: Q (and K, unless V aliases it) back in place as bf16, K
 // and V into the cache at slot(pos) in the cache's element type.  HBM-bound by construction:
 // every byte moves once; at 256 canvas rows the launch is a few megabytes, i.e. latency-bound.
 #include "attn_params.h"
@@ -102,10 +102,12 @@ __device__ __forceinline__ uint16_t cache_bits(uint32_t dt, float v) {
 template <int PER>
 __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   __shared__ float stage[4][512];
+  __shared__ float cos_t[256], sin_t[256];
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const uint32_t tok = blockIdx.x, h = blockIdx.y * 4 + wave;
+  const uint32_t tok = blockIdx.x, h_raw = blockIdx.y * 4 + wave;
   const uint32_t n_heads = p.hq + 2 * p.hkv;
-  if (h >= n_heads) return;   // the whole wave leaves; nothing below synchronises across waves
+  const bool head_ok = h_raw < n_heads;
+  const uint32_t h = head_ok ? h_raw : n_heads - 1u;   // (a wave without a head of its own stays for the barrier below)
   const uint32_t hd = p.hd;
   const bool is_q = h < p.hq, is_k = !is_q && h < p.hq + p.hkv;
   const uint32_t hh = is_q ? h : (h - p.hq) % p.hkv;
@@ -122,6 +124,19 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   const bool active = d0 < hd;
   float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (active) load_row<PER>(src + d0, x);
+  // The angles depend on the position only: the workgroup's four heads share one table of cos and sin,
+  // one pair per thread, worked out while the rows are on their way (rotation, cpu.rs:31-65: pairs
+  // (d, hd/2 + d) for d < rot/2; split-half: rot = hd, theta 1e4; proportional: rot = hd/4, theta 1e6,
+  // everything else is left alone).
+  const uint32_t half_rot = p.is_full ? hd / 8 : hd / 2, off = hd / 2;
+  if (threadIdx.x < half_rot) {
+    float sn, cs;
+    sincosf((float)pos * p.inv_freq[threadIdx.x], &sn, &cs);
+    cos_t[threadIdx.x] = cs;
+    sin_t[threadIdx.x] = sn;
+  }
+  __syncthreads();
+  if (!head_ok) return;   // the whole wave leaves; nothing below synchronises across waves
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) ss += x[i] * x[i];
@@ -149,13 +164,9 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   }
   __builtin_amdgcn_wave_barrier();   // the stage is private to the wave, whose LDS operations execute in order
 
-  // rotation (cpu.rs:31-65): pairs (d, hd/2 + d) for d < rot/2; split-half: rot = hd, theta 1e4;
-  // proportional: rot = hd/4, theta 1e6, everything else is left alone.  One pair per lane and pass.
-  const uint32_t half_rot = p.is_full ? hd / 8 : hd / 2, off = hd / 2;
+  // one pair per lane and pass
   for (uint32_t dd = lane; dd < half_rot; dd += 64) {
-    const float a = (float)pos * p.inv_freq[dd];
-    float s, c;
-    sincosf(a, &s, &c);
+    const float s = sin_t[dd], c = cos_t[dd];
     const float x0 = st[dd], x1 = st[dd + off];
     st[dd] = x0 * c - x1 * s;
     st[dd + off] = x0 * s + x1 * c;
