@@ -38,6 +38,8 @@ def parse_args():
     ap.add_argument("--streamed-merge", action="store_true",
                     help="merge split partial rows with the streaming kernel even where the up-front one would be picked")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kv-from-hbm", action="store_true",
+                    help="skip the extra measurement with the cache rows coming from HBM (keeps a profile to one kind of launch)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline sample time")
     ap.add_argument("--check-toks", type=int, default=12)
     ap.add_argument("--calib-copy-mib", type=int, default=0,
@@ -662,7 +664,7 @@ def main():
     # hint for this situation (DG_ATTN_F_KV_FROM_HBM).  Reported beside the metric, not as the metric. ----
     kv_from_hbm = None
     kv_alloc_bytes = kd.numel() * kd.element_size()
-    if w.head_dim == 512 and 32e6 <= kv_alloc_bytes <= 256e6 and ms_per_step > 0.1:
+    if not args.no_kv_from_hbm and w.head_dim == 512 and 32e6 <= kv_alloc_bytes <= 256e6 and ms_per_step > 0.1:
         n_copies = int(min(16, -(-600e6 // kv_alloc_bytes)))
         copies = [kd] + [kd.clone() for _ in range(n_copies - 1)]
         kv_from_hbm = {"copies": n_copies, "cache_bytes": int(kv_alloc_bytes)}
