@@ -455,11 +455,13 @@ def test_f16_cache_with_bf16_queries(gpu_ready, po):
                      max_abs=2e-3, mean_abs=1e-4)
 
 
-def test_ring_cache_and_region_offset(gpu_ready, po):
-    """Sliding layer on a wrapped power-of-two ring placed at a non-zero region offset."""
+@pytest.mark.parametrize("hq,hkv,hd,flags", [(16, 8, 256, 0), (16, 2, 512, capi.DG_ATTN_F_KV_FROM_HBM)])
+def test_ring_cache_and_region_offset(gpu_ready, po, hq, hkv, hd, flags):
+    """Sliding layer on a wrapped power-of-two ring placed at a non-zero region offset (also at head_dim
+    512 with the instance that touches tiles ahead of their loads: the touches stay inside the ring)."""
     import torch
     rng = np.random.default_rng(31)
-    c, hq, hkv, hd, kvl, window, ring = 256, 16, 8, 256, 5000, 1024, 2048
+    c, kvl, window, ring = 256, 5000, 1024, 2048
     t_all = kvl + c
     row = 2 * hkv * hd
     q = rng.standard_normal((c, hq, hd)).astype(np.float32)
@@ -472,7 +474,7 @@ def test_ring_cache_and_region_offset(gpu_ready, po):
     region = 4096
     buf = np.concatenate([np.full(region // 2, 0x7E00, np.uint16), ringbits.ravel()])
     d = A.make_desc(c, hq, hkv, hd, kvl, window=window, kv_ring_mask=ring - 1, q_dtype=capi.DG_BF16,
-                    kv_dtype=capi.DG_F16, out_dtype=capi.DG_F32, kv_region_bytes=region)
+                    kv_dtype=capi.DG_F16, out_dtype=capi.DG_F32, kv_region_bytes=region, flags=flags)
     out = torch.zeros(c * hq * hd, dtype=torch.float32, device="cuda")
     lse = torch.zeros(c * hq, dtype=torch.float32, device="cuda")
     A.forward(d, A.to_device_bits(qb), A.to_device_bits(buf), out, lse, A.alloc_workspace(d))
