@@ -562,7 +562,7 @@ def main():
 
     # ---- HIP graphs of the step: `round_len` steps for the timed rounds (a denoise loop replays its
     # layers the same way, so host launch latency is not in the measurement), 50 steps for settling ----
-    round_len = max(1, min(50, args.steps // 2))   # (few steps: two rounds, so that graph launches stay a small part)
+    round_len = max(1, min(50, args.steps))   # (few steps: one graph of them all, its launch is then paid once)
     n_rounds, rem = divmod(args.steps, round_len)
     graph = settle_graph = None
     if not args.eager:
