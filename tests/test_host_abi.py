@@ -31,6 +31,16 @@ def test_library_exports_every_declared_symbol():
     assert lib.dg_attn_abi_version() == 1
 
 
+def test_flag_constants_match_the_header():
+    """The ctypes binding spells the desc.flags bits out again: they must be the header's."""
+    text = open(os.path.join(ROOT, "include", "dg_attn.h")).read()
+    defs = dict(re.findall(r"#define\s+(DG_ATTN_F_[A-Z0-9_]+)\s+(0x[0-9a-fA-F]+)u?", text))
+    assert len(defs) >= 7
+    for name, value in defs.items():
+        assert getattr(capi, name) == int(value, 16), name
+    assert len(set(defs.values())) == len(defs)          # no two flags share a bit
+
+
 def test_reference_struct_sizes():
     assert C.sizeof(capi.LayerOffsets) == 200     # 23 u64 + 4 u32, repr(C)
     assert C.sizeof(capi.StepParams) == 48
