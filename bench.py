@@ -86,6 +86,7 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     "cfg3_global": (152.5e6 + 33.8e6, "profiles/attn_mfma_kernel_cfg3_global_hbm_traffic.md"),
     "cfg4_long": (555.3e6 + 33.8e6, "profiles/attn_mfma_kernel_cfg4_long_hbm_traffic.md"),
+    "cfg2_sliding": (12.9e6 + 12.8e6, "profiles/attn_mfma_kernel_cfg2_sliding_kernel_trace.md"),
 }
 
 
