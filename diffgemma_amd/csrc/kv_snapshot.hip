@@ -57,8 +57,11 @@ __global__ void __launch_bounds__(256) kv_move_kernel(const MoveParams p) {
                             : (int64_t)slot * L.k_tok_b + (int64_t)head * L.k_head_b) +
                      (uint64_t)w * 16u;
     char* in_blob = p.blob + L.blob_off + row * L.row_bytes + (uint64_t)w * 16u;
-    if (p.to_blob) *(uint4*)in_blob = *(const uint4*)in_cache;
-    else *(uint4*)in_cache = *(const uint4*)in_blob;
+    // every byte is touched once: non-temporal loads and stores, so that the stream does not push
+    // through the L2s what it will not read again (gather + scatter of the 30-layer cache: 0.791 -> 0.765 ms)
+    typedef uint32_t mv_u32x4 __attribute__((ext_vector_type(4)));
+    if (p.to_blob) __builtin_nontemporal_store(__builtin_nontemporal_load((const mv_u32x4*)in_cache), (mv_u32x4*)in_blob);
+    else __builtin_nontemporal_store(__builtin_nontemporal_load((const mv_u32x4*)in_blob), (mv_u32x4*)in_cache);
   }
 }
 
