@@ -381,14 +381,16 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
   const uint32_t hull_hi = rb.extra < p.t_all ? p.t_all : min(rb.hi, p.t_all);
 
   // f(position, score) for every visible key of the row; each thread takes one float4 out of
-  // every 256 and has four of them in flight
+  // every 256 and has four of them in flight.  The plane is read once: non-temporal loads (here and
+  // for the sample above), so that 135 MB of scores per block do not push the V rows, which every
+  // row of a KV group gathers from, out of the L2s (whole call 0.715 -> 0.664 ms)
   auto scan_row = [&](auto&& f) {
     for (uint32_t t4 = hull_lo + 4u * tid; t4 < hull_hi; t4 += 4096u) {
       f32x4 v[4];
 #pragma unroll
       for (uint32_t u = 0; u < 4; ++u) {
         const uint32_t a = t4 + 1024u * u;
-        v[u] = a < hull_hi ? *(const f32x4*)(srow + a) : f32x4{0.f, 0.f, 0.f, 0.f};
+        v[u] = a < hull_hi ? __builtin_nontemporal_load((const f32x4*)(srow + a)) : f32x4{0.f, 0.f, 0.f, 0.f};
       }
 #pragma unroll
       for (uint32_t u = 0; u < 4; ++u) {
@@ -423,7 +425,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(const TopkParams tp) {
 #pragma unroll
       for (uint32_t u = 0; u < 8; ++u) {      // m <= 2048: eight samples per thread, all in flight
         const uint32_t i = tid + 256u * u;
-        sv[u] = i < m ? srow[hull_lo + i * stride] : 0.f;
+        sv[u] = i < m ? __builtin_nontemporal_load(srow + hull_lo + i * stride) : 0.f;
       }
 #pragma unroll
       for (uint32_t u = 0; u < 8; ++u) {
