@@ -279,14 +279,16 @@ def test_both_merge_kernels_give_the_same_bits(gpu_ready, hd, hq, hkv, splits, c
     assert np.isfinite(a_lse).all() and np.any(a != 0)
 
 
+@pytest.mark.parametrize("layout", ["head_major", "reference"])
 @pytest.mark.parametrize("canvas,hq,hkv,kv_len,splits", [(256, 16, 2, 32768, 0), (64, 16, 2, 1000, 0), (100, 8, 1, 2049, 3),
                                                          (33, 8, 2, 70, 1), (256, 16, 2, 4099, 8)])
-def test_kv_from_hbm_hint_changes_no_bit(gpu_ready, canvas, hq, hkv, kv_len, splits):
+def test_kv_from_hbm_hint_changes_no_bit(gpu_ready, canvas, hq, hkv, kv_len, splits, layout):
     """DG_ATTN_F_KV_FROM_HBM selects the head_dim 512 kernel that touches key/value tiles into the L2 ahead
     of their loads: a change in timing only.  Ragged last tiles, splits shorter than the look-ahead and a
-    single tile included."""
+    single tile included, with key rows contiguous per head and in the reference's slot-major layout (rows of
+    a tile a whole slot apart)."""
     import torch
-    w = W.Workload("hint", canvas, hq, hkv, 512, kv_len, causal_rows=canvas // 2, seed=17)
+    w = W.Workload("hint", canvas, hq, hkv, 512, kv_len, causal_rows=canvas // 2, seed=17, layout=layout)
     q, kv = W.generate(w)
     qd, kd = W.device_arrays(w, q, kv)
 
