@@ -17,9 +17,12 @@ DG_ATTN_F_F32_PARTIALS = 0x8
 DG_ATTN_F_F16_PARTIALS = 0x10
 DG_ATTN_F_STREAMED_MERGE = 0x20
 DG_ATTN_F_KV_FROM_HBM = 0x40
-DG_DBG_ATTN_NONPOSITIVE_L = 1
-DG_DBG_ATTN_NONFINITE_OUT = 2
-DG_DBG_KERNEL_ATTENTION = 7
+# the reference's DebugStatus vocabulary (debug_status.metal:8-19, dgq_kernels.metal:33-34)
+DG_DBG_ERR_SOFTMAX_NORM_ZERO = 3
+DG_DBG_ERR_NONFINITE = 4
+DG_DBG_ERR_BAD_DIM = 8
+DG_DBG_KERNEL_QK_ROPE_KV = 25
+DG_DBG_KERNEL_ATTENTION = 26
 
 DG_ROPE_F_QK_TRUNCATE = 0x1
 

@@ -88,7 +88,7 @@ __global__ void __launch_bounds__(64) attn_scalar_kernel(const AttnParams p, con
     }
   }
   if (lane == 0) {
-    if (!(l > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l));
+    if (!(l > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, (tok << 16) | qh, (tok << 16) | qh);
     if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l > 0.f ? m * kLn2 + logf(l) : -INFINITY;
   }
 #pragma unroll
@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(64) attn_scalar_kernel(const AttnParams p, con
     const uint32_t d = lane + 64u * i;
     if (d < hd) {
       const float y = l > 0.f ? acc[i] / l : 0.f;
-      if (p.dbg && nonfinite(y)) dbg_report(p.dbg, 2u, (tok << 16) | qh, d);
+      if (p.dbg && nonfinite(y)) dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_ATTENTION, (tok << 16) | qh, d);
       store_out(p, qoff + d, y);
     }
   }
@@ -175,7 +175,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
         bool bad = false;
 #pragma unroll
         for (int e = 0; e < 8; ++e) bad = bad || nonfinite(acc[e]);
-        if (bad) dbg_report(p.dbg, 2u, (tok << 16) | qh, d8 * 8u);
+        if (bad) dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_ATTENTION, (tok << 16) | qh, d8 * 8u);
       }
       if (p.out_dtype == DT_BF16) {   // eight bf16 in one 16-byte store
         const bool tr = p.out_trunc != 0;
@@ -192,7 +192,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
       }
     }
     if (lane == 0) {
-      if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));
+      if (!(den > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, (tok << 16) | qh, (tok << 16) | qh);
       if (p.lse) p.lse[(size_t)tok * p.hq + qh] = den > 0.f ? mx * kLn2 + logf(den) : -INFINITY;
     }
     return;
@@ -225,7 +225,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
     }
     if (!live) continue;
     if (p.dbg && (nonfinite(o.x) || nonfinite(o.y) || nonfinite(o.z) || nonfinite(o.w)))
-      dbg_report(p.dbg, 2u, (tok << 16) | qh, d4 * 4u);
+      dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_ATTENTION, (tok << 16) | qh, d4 * 4u);
     if (p.out_dtype == DT_F32) {
       const wt_u32x4 o4 = {__float_as_uint(o.x), __float_as_uint(o.y), __float_as_uint(o.z), __float_as_uint(o.w)};
       wt_store16(wt_window_wave((const float*)p.out + ooff), d4 * 16u, o4);
@@ -244,7 +244,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnParams p, con
     }
   }
   if (lane == 0) {
-    if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));
+    if (!(den > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, (tok << 16) | qh, (tok << 16) | qh);
     if (p.lse) p.lse[(size_t)tok * p.hq + qh] = den > 0.f ? mx * kLn2 + logf(den) : -INFINITY;
   }
 }
@@ -308,7 +308,7 @@ __global__ void __launch_bounds__(256) attn_merge_few_kernel(const AttnParams p,
       bool bad = false;
 #pragma unroll
       for (int e = 0; e < 8; ++e) bad = bad || nonfinite(acc[e]);
-      if (bad) dbg_report(p.dbg, 2u, (tok << 16) | qh, d8 * 8u);
+      if (bad) dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_ATTENTION, (tok << 16) | qh, d8 * 8u);
     }
     if (p.out_dtype == DT_BF16) {
       const bool tr = p.out_trunc != 0;
@@ -323,7 +323,7 @@ __global__ void __launch_bounds__(256) attn_merge_few_kernel(const AttnParams p,
     }
   }
   if (lane == 0) {
-    if (!(den > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(den));
+    if (!(den > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, (tok << 16) | qh, (tok << 16) | qh);
     if (p.lse) p.lse[(size_t)tok * p.hq + qh] = den > 0.f ? mx * kLn2 + logf(den) : -INFINITY;
   }
 }
@@ -504,7 +504,7 @@ __global__ void __launch_bounds__(256) attn_state_merge_kernel(const StateMergeP
     }
     o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
     if (p.dbg && (nonfinite(o.x) || nonfinite(o.y) || nonfinite(o.z) || nonfinite(o.w)))
-      dbg_report(p.dbg, 2u, ((row / p.hq) << 16) | (row % p.hq), d);
+      dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_ATTENTION, ((row / p.hq) << 16) | (row % p.hq), d);
     if (p.state_out) *(float4*)(p.state_out + acc0 + d) = o;
     if (p.out) {
       const size_t idx = (size_t)row * p.hd + d;
@@ -524,7 +524,7 @@ __global__ void __launch_bounds__(256) attn_state_merge_kernel(const StateMergeP
   }
   if (lane == 0) {
     const float lse = den > 0.f ? mx + __logf(den) : -INFINITY;
-    if (p.dbg && p.out && !(den > 0.f)) dbg_report(p.dbg, 1u, ((row / p.hq) << 16) | (row % p.hq), __float_as_uint(den));
+    if (p.dbg && p.out && !(den > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, ((row / p.hq) << 16) | (row % p.hq), ((row / p.hq) << 16) | (row % p.hq));
     if (p.lse) p.lse[row] = lse;
     if (p.state_out) {
       p.state_out[row] = lse;

@@ -711,7 +711,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
       wt_store8(wt_window(p.part_ml + wg_prow0 * 2), (r - row0) * 8u, ml2);
     } else if (row_ok) {
       if (p.lse) p.lse[(size_t)tok * p.hq + qh] = l_tot > 0.f ? m_pub * kLn2 + __logf(l_tot) : -INFINITY;
-      if (p.dbg && !(l_tot > 0.f)) dbg_report(p.dbg, 1u, (tok << 16) | qh, __float_as_uint(l_tot));
+      if (p.dbg && !(l_tot > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, (tok << 16) | qh, (tok << 16) | qh);
     }
   }
   __syncthreads();
@@ -792,7 +792,7 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
         const float y2 = x[2] * inv, y3 = x[3] * inv;
         const size_t idx = idx0 + 8 * q4;
         if (p.dbg && !(fabsf(y0) + fabsf(y1) + fabsf(y2) + fabsf(y3) <= 3.402823466e38f))   // NaN or infinity
-          dbg_report(p.dbg, 2u, (tok_o << 16) | qh_o, 32u * (dgrp * NDBW + i) + 4u * g2 + 8u * q4);
+          dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_ATTENTION, (tok_o << 16) | qh_o, 32u * (dgrp * NDBW + i) + 4u * g2 + 8u * q4);
         if (p.out_dtype == DT_F32) {
           f32x4 v4 = {y0, y1, y2, y3};
           *(f32x4*)((float*)p.out + idx) = v4;

@@ -120,11 +120,24 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f, bool trunc) {
   return (uint16_t)(u >> 16);
 }
 
-// first-writer-wins status record, like the reference's DebugStatus buffer
-__device__ __forceinline__ void dbg_report(uint32_t* dbg, uint32_t code, uint32_t tg, uint32_t value) {
+// The reference's DebugStatus vocabulary (src/shaders/include/debug_status.metal:8-19 error codes,
+// src/shaders/include/dgq_kernels.metal:33-34 kernel ids), decoded on the host by
+// src/metal/debug_status.rs:33-75.  include/dg_attn.h carries the same numbers as DG_DBG_*.
+enum : uint32_t {
+  DBG_ERR_SOFTMAX_NORM_ZERO = 3u,   // a row's softmax denominator was not > 0; value = (tok << 16) | query head
+  DBG_ERR_NONFINITE = 4u,           // a result was NaN or infinite; value = element index (attention) / canvas row (producer)
+  DBG_ERR_BAD_DIM = 8u,
+  DBG_KERNEL_QK_ROPE_KV = 25u,
+  DBG_KERNEL_ATTENTION = 26u,
+};
+
+// first-writer-wins status record, like the reference's debug_set_error (debug_status.metal:38-52).
+// tg is (tok << 16) | query head of the row at fault (the reference's call sites pass 0 there).
+__device__ __forceinline__ void dbg_report(uint32_t* dbg, uint32_t code, uint32_t kernel_id, uint32_t tg,
+                                           uint32_t value) {
   if (dbg == nullptr) return;
   if (atomicCAS(dbg, 0u, code) == 0u) {
-    dbg[1] = 7u;
+    dbg[1] = kernel_id;
     dbg[2] = tg;
     dbg[3] = value;
   }

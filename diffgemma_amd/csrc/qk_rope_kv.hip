@@ -143,7 +143,7 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)hd + kRmsEps);
   if (lane == 0 && !(inv == inv && fabsf(inv) != INFINITY))
-    dbg_report(p.dbg, DG_DBG_ROPE_NONFINITE, (tok << 16) | h, __float_as_uint(inv));
+    dbg_report(p.dbg, DBG_ERR_NONFINITE, DBG_KERNEL_QK_ROPE_KV, (tok << 16) | h, tok);   // (qk_rope_kv.metal:77: tag = canvas row)
 
   uint16_t bits[8];
   if (!is_q && !is_k) {   // V: normalise without weight, write to the cache (cpu.rs:110-122)

@@ -219,10 +219,25 @@ typedef struct dg_debug_status {
   uint32_t code, kernel_id, tg_id, value;
 } dg_debug_status;
 
-#define DG_DBG_ATTN_NONPOSITIVE_L 1u  /* a row's softmax denominator was not > 0 */
-#define DG_DBG_ATTN_NONFINITE_OUT 2u  /* an output element was NaN/inf (tg_id = token << 16 | query
-                                         head, value = head_dim index of the group of elements) */
-#define DG_DBG_KERNEL_ATTENTION 7u
+/* The record a kernel leaves in *dbg is the reference's own, so that the host-side decoder it already has
+ * (check_status, src/metal/debug_status.rs:33-75) names the right error in the right kernel: error codes
+ * DbgErrorCode (src/shaders/include/debug_status.metal:8-19), kernel ids DbgKernelId
+ * (src/shaders/include/dgq_kernels.metal:33-34).  First writer wins (debug_status.metal:38-52).
+ *   code 3, kernel 26: a row's softmax denominator was not > 0; value = (canvas row << 16) | query head
+ *                      (attention.metal:123, attention_mma2.metal:283, attention_mma_full.metal:371)
+ *   code 4, kernel 26: an output element was NaN or infinite; value = its index in the head (of the first
+ *                      element of the group a lane stores; attention.metal:129, attention_mma_full.metal:384-389)
+ *   code 4, kernel 25: the producer found a head whose 1/rms was not finite; value = canvas row
+ *                      (qk_rope_kv.metal:77)
+ * tg_id is (canvas row << 16) | head of the row at fault in all three (the reference's call sites leave 0).
+ * Code 8 (DbgErrBadDim, qk_rope_kv.metal:48) is never written: head_dim is validated on the host and a bad
+ * one is DG_ERR_SHAPE before anything is enqueued.  The top-k entry points take dbg and write nothing: the
+ * reference's top-k kernels assert nothing either (attention_topk.metal has no debug_set_error). */
+#define DG_DBG_ERR_SOFTMAX_NORM_ZERO 3u
+#define DG_DBG_ERR_NONFINITE 4u
+#define DG_DBG_ERR_BAD_DIM 8u
+#define DG_DBG_KERNEL_QK_ROPE_KV 25u
+#define DG_DBG_KERNEL_ATTENTION 26u
 
 /* One layer's attention with exactly the buffers encode_layer_attention_dispatch binds:
  * q = arena+attnq_off (bf16 [canvas][16][hd]), kvcache = whole KV buffer (f16, the kernel adds
@@ -322,9 +337,6 @@ int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* 
  * the reference's truncating bf16 store, the cache as f16 (kv_store). */
 int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
                            const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream);
-
-#define DG_DBG_ROPE_NONFINITE 3u        /* a head's 1/rms was not finite */
-#define DG_DBG_KERNEL_QK_ROPE_KV 6u
 
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);

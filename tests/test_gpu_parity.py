@@ -526,7 +526,8 @@ def test_debug_status_reports_nonfinite_output(gpu_ready, fixture):
     bad = A.AttnRig.from_fixture(A.Fixture(q=f.q, kvcache=kv, layer=f.layer, canvas=f.canvas, n_q_heads=f.n_q_heads, kv_len=f.kv_len))
     bad.run_dispatch(causal=0)
     st = bad.read_debug_status()
-    assert (st.code, st.kernel_id) == (capi.DG_DBG_ATTN_NONFINITE_OUT, capi.DG_DBG_KERNEL_ATTENTION)
+    # DbgErrNonFinite = 4 in DbgKernelAttention = 26: what the reference's check_status decodes
+    assert (st.code, st.kernel_id) == (4, 26) == (capi.DG_DBG_ERR_NONFINITE, capi.DG_DBG_KERNEL_ATTENTION)
     tok, head = st.tg_id >> 16, st.tg_id & 0xffff
     assert tok < f.canvas and head < f.n_q_heads // nkv       # a head of the group that reads KV head 0
     assert st.value <= 3 < st.value + 8

@@ -72,6 +72,24 @@ def test_layer_shapes(gpu_ready, po, shape):
     assert ds[0] == 0, f"debug status {ds}"
 
 
+def test_debug_status_names_the_producer(gpu_ready):
+    """A NaN in one head's input makes that head's 1/rms non-finite; the record the kernel leaves is the
+    reference's: DbgErrNonFinite = 4 in DbgKernelQkRopeKv = 25, value = the canvas row
+    (qk_rope_kv.metal:77; decoded by src/metal/debug_status.rs:33-75).  (An infinity would not do: the sum of
+    squares is then +inf and 1/sqrt(+inf) = 0 is finite, in the reference too.)"""
+    f = QR.random_fixture(8, 4, 2, 64, 40, is_full=False, v_proj=1, seed=3)
+    clean = QR.RopeRig(f)
+    clean.run_dispatch()
+    assert clean.buf_dbg.cpu().numpy().view(np.uint32)[0] == 0
+    tok, head = 5, 3
+    f.q[(tok * f.n_q_heads + head) * f.head_dim + 7] = np.float32(np.nan)
+    bad = QR.RopeRig(f)
+    bad.run_dispatch()
+    code, kernel_id, tg_id, value = (int(x) for x in bad.buf_dbg.cpu().numpy().view(np.uint32))
+    assert (code, kernel_id) == (4, 25) == (capi.DG_DBG_ERR_NONFINITE, capi.DG_DBG_KERNEL_QK_ROPE_KV)
+    assert value == tok and tg_id == (tok << 16) | head
+
+
 def test_write_suppression_and_untouched_rows(gpu_ready, po):
     """kv_write_end (qk_rope_kv.metal:56-60): pad rows are normed and rotated in place but never reach
     the cache; every slot the launch does not own keeps its bits."""

@@ -41,6 +41,30 @@ def test_flag_constants_match_the_header():
     assert len(set(defs.values())) == len(defs)          # no two flags share a bit
 
 
+def test_debug_status_vocabulary_is_the_references():
+    """The numbers the reference's host side decodes (src/metal/debug_status.rs:33-75): DbgErrorCode of
+    src/shaders/include/debug_status.metal:8-19 and DbgKernelId of src/shaders/include/dgq_kernels.metal:33-34."""
+    want = {"DG_DBG_ERR_SOFTMAX_NORM_ZERO": 3, "DG_DBG_ERR_NONFINITE": 4, "DG_DBG_ERR_BAD_DIM": 8,
+            "DG_DBG_KERNEL_QK_ROPE_KV": 25, "DG_DBG_KERNEL_ATTENTION": 26}
+    text = open(os.path.join(ROOT, "include", "dg_attn.h")).read()
+    defs = {k: int(v) for k, v in re.findall(r"#define\s+(DG_DBG_[A-Z0-9_]+)\s+(\d+)u", text)}
+    assert defs == want
+    for name, value in want.items():
+        assert getattr(capi, name) == value, name
+    # the kernels' own spelling of the same numbers
+    src = open(os.path.join(ROOT, "diffgemma_amd", "csrc", "attn_params.h")).read()
+    dev = {k: int(v) for k, v in re.findall(r"(DBG_(?:ERR|KERNEL)_[A-Z0-9_]+) = (\d+)u", src)}
+    assert dev == {k[3:]: v for k, v in want.items()}
+    # no kernel source writes a literal code or kernel id
+    for f in os.listdir(os.path.join(ROOT, "diffgemma_amd", "csrc")):
+        body = open(os.path.join(ROOT, "diffgemma_amd", "csrc", f)).read()
+        for call in re.findall(r"dbg_report\(([^;]*)\);", body):
+            if "uint32_t* dbg" in call:
+                continue
+            args = [a.strip() for a in call.split(",")]
+            assert args[1].startswith("DBG_ERR_") and args[2].startswith("DBG_KERNEL_"), (f, call)
+
+
 def test_reference_struct_sizes():
     assert C.sizeof(capi.LayerOffsets) == 200     # 23 u64 + 4 u32, repr(C)
     assert C.sizeof(capi.StepParams) == 48
