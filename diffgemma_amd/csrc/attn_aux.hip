@@ -478,29 +478,42 @@ __global__ void __launch_bounds__(256) attn_state_merge_kernel(const StateMergeP
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t row = blockIdx.x * 4 + wave;
   if (row >= p.rows) return;
+  // The (m, l) pairs of the row are read once, before anything is written: state_out may be one of the
+  // inputs, and lane 0 overwrites the row's (m, l) there at the end.  Every lane derives the same
+  // weights from them and keeps them in registers for the accumulator loop.
+  float w[kMaxStates], lw[kMaxStates];
   float mx = -INFINITY;
-  for (uint32_t i = 0; i < p.n; ++i) {
-    const float2 ml = make_float2(p.states[i][row], p.states[i][p.rows + row]);
-    if (ml.y > 0.f) mx = fmaxf(mx, ml.x);
+#pragma unroll
+  for (uint32_t i = 0; i < kMaxStates; ++i) {
+    w[i] = -INFINITY;   // the exponent m for now; a state that saw no key of the row does not count
+    lw[i] = 0.f;
+    if (i < p.n) {
+      const float m_i = p.states[i][row], l_i = p.states[i][p.rows + row];
+      if (l_i > 0.f) {
+        w[i] = m_i;
+        lw[i] = l_i;
+      }
+    }
+    mx = fmaxf(mx, w[i]);
   }
   float den = 0.f;
-  for (uint32_t i = 0; i < p.n; ++i) {
-    const float2 ml = make_float2(p.states[i][row], p.states[i][p.rows + row]);
-    if (ml.y > 0.f) den += ml.y * __expf(ml.x - mx);
+#pragma unroll
+  for (uint32_t i = 0; i < kMaxStates; ++i) {
+    w[i] = lw[i] > 0.f ? __expf(w[i] - mx) : 0.f;   // weight of the state's accumulators
+    den += lw[i] * w[i];
   }
   const float inv = den > 0.f ? 1.f / den : 0.f;
   const size_t acc0 = state_acc_offset(p.rows) + (size_t)row * p.hd;
   for (uint32_t d = lane * 4u; d < p.hd; d += 256u) {
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t i = 0; i < p.n; ++i) {
-      const float2 ml = make_float2(p.states[i][row], p.states[i][p.rows + row]);
-      if (!(ml.y > 0.f)) continue;
-      const float w = __expf(ml.x - mx);
+#pragma unroll
+    for (uint32_t i = 0; i < kMaxStates; ++i) {
+      if (i >= p.n || lw[i] == 0.f) continue;   // the same in every lane
       const float4 a = *(const float4*)(p.states[i] + acc0 + d);
-      o.x = __builtin_fmaf(w, a.x, o.x);
-      o.y = __builtin_fmaf(w, a.y, o.y);
-      o.z = __builtin_fmaf(w, a.z, o.z);
-      o.w = __builtin_fmaf(w, a.w, o.w);
+      o.x = __builtin_fmaf(w[i], a.x, o.x);
+      o.y = __builtin_fmaf(w[i], a.y, o.y);
+      o.z = __builtin_fmaf(w[i], a.z, o.z);
+      o.w = __builtin_fmaf(w[i], a.w, o.w);
     }
     o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
     if (p.dbg && (nonfinite(o.x) || nonfinite(o.y) || nonfinite(o.z) || nonfinite(o.w)))
@@ -524,7 +537,8 @@ __global__ void __launch_bounds__(256) attn_state_merge_kernel(const StateMergeP
   }
   if (lane == 0) {
     const float lse = den > 0.f ? mx + __logf(den) : -INFINITY;
-    if (p.dbg && p.out && !(den > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, ((row / p.hq) << 16) | (row % p.hq), ((row / p.hq) << 16) | (row % p.hq));
+    const uint32_t tag = ((row / p.hq) << 16) | (row % p.hq);
+    if (p.dbg && p.out && !(den > 0.f)) dbg_report(p.dbg, DBG_ERR_SOFTMAX_NORM_ZERO, DBG_KERNEL_ATTENTION, tag, tag);
     if (p.lse) p.lse[row] = lse;
     if (p.state_out) {
       p.state_out[row] = lse;

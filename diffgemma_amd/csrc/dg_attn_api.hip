@@ -690,12 +690,27 @@ int dg_attention_block_state_bytes(const dg_layer_offsets* L, const dg_attn_dims
   if (!L || !dims || !out_bytes) return DG_ERR_NULL;
   dg_attn_desc d;
   desc_from_reference(L, dims, kv_len, &d);
-  size_t ws_full = 0, ws_part = 0;
+  size_t ws_full = 0;
   int rc = dg_attn_workspace_bytes(&d, &ws_full);
   if (rc != DG_OK) return rc;
-  // a block's partial never needs more than the partial of the whole range (fewer key tiles: fewer splits)
-  rc = dg_attn_partial_workspace_bytes(&d, 0u, d.kv_len + d.canvas, &ws_part);
+  // The partial of a block [a, b) is split over workgroups like a whole call, and the number of splits a
+  // range resolves to is not monotone in its length (ceil(n / ceil(n / s)) jumps up and down with n), so a
+  // shorter range can take more splits than the whole one.  What bounds every range is the cap the split
+  // count is cut to before that rounding; the partial workspace is sized for it, with fp32 partial rows
+  // (a partial's result is fp32 accumulators).
+  const dg_attn_desc pd = partial_desc(&d);
+  Plan pl;
+  const int cus = plan_cus();
+  rc = make_plan(&pd, cus, &pl);
   if (rc != DG_OK) return rc;
+  const uint32_t ntiles_full = std::max(1u, (pl.t_all + dg::kBlockN - 1) / dg::kBlockN);
+  const uint32_t base = d.n_kv_heads * pl.n_mtiles;
+  const uint32_t cap = std::min(std::min(std::max(1u, (uint32_t)cus / std::max(1u, base)), std::max(1u, ntiles_full / 6u)),
+                                kMaxSplits);
+  size_t ws_part = 0;
+  if (cap > 1)
+    ws_part = align_up((size_t)cap * d.n_kv_heads * pl.rows_pad * d.head_dim * 4) +
+              align_up((size_t)cap * d.n_kv_heads * pl.rows_pad * 2 * 4);
   *out_bytes = 2 * align_up(state_bytes_of(&d)) + std::max(ws_full, ws_part);
   return DG_OK;
 }

@@ -13,13 +13,12 @@ iterations from `seed + iteration`, the prefix rows of the caches stay.
 from __future__ import annotations
 
 import ctypes as C
-import time
 from dataclasses import dataclass, field
 from typing import List, Optional
 
 import numpy as np
 
-from . import attention as A, attention_topk as T, capi, qk_rope_kv as QR, rounding as R, step_kv
+from . import attention as A, attention_topk as T, capi, qk_rope_kv as QR, step_kv
 
 
 @dataclass
@@ -40,6 +39,7 @@ class ScheduleLayer:
     q_norm_w: object
     k_norm_w: object
     out: object
+    lse: object             # [canvas][n_q_heads] fp32 log-sum-exp of the row's scores (dense layers)
     workspace: object
     flops: float = 0.0
 
@@ -101,6 +101,7 @@ class DenoiseSchedule:
                 q_norm_w=A.to_device_bits(R.f32_to_bf16_bits_rne(f.q_norm_w)),
                 k_norm_w=A.to_device_bits(R.f32_to_bf16_bits_rne(f.k_norm_w)),
                 out=torch.zeros(canvas * nq * hd, dtype=torch.int16, device="cuda"),
+                lse=torch.zeros(canvas * nq, dtype=torch.float32, device="cuda"),
                 workspace=A.alloc_workspace(ad),
                 flops=capi.visible_pairs(ad)[1])
             if full and self.global_topk and self.topk_ws is None:
@@ -127,7 +128,7 @@ class DenoiseSchedule:
             if lay.full and self.global_topk:
                 T.forward(lay.attn_desc, self.k_cfg, lay.q, lay.cache, lay.out, self.topk_ws)
             else:
-                A.forward(lay.attn_desc, lay.q, lay.cache, lay.out, None, lay.workspace)
+                A.forward(lay.attn_desc, lay.q, lay.cache, lay.out, lay.lse, lay.workspace)
 
     def run_eager(self) -> None:
         """One iteration as plain launches on a side stream (the stream a capture would use)."""
@@ -150,26 +151,3 @@ class DenoiseSchedule:
 
     def outputs(self):
         return [lay.out.clone() for lay in self.layers]
-
-    def oracle_check(self, po, layer_index: int, toks) -> dict:
-        """Layer `layer_index`'s output rows `toks` against the CPU oracle, on the inputs the device
-        holds after the producer ran (rotated q, cache with the canvas rows written)."""
-        lay = self.layers[layer_index]
-        canvas, nq = self.canvas, self.n_q_heads
-        qh = R.bf16_bits_to_f32(lay.q.cpu().numpy().view(np.uint16))
-        kvh = R.bf16_bits_to_f32(lay.cache.cpu().numpy().view(np.uint16))
-        od = po.make_desc(canvas, nq, lay.n_kv_heads, lay.head_dim, self.kv_len, window=lay.window,
-                          kv_ring_mask=lay.ring_mask, layout="head_major", t_cap=lay.slots)
-        toks = np.asarray(toks, dtype=np.uint32)
-        t0 = time.perf_counter()
-        if lay.full and self.global_topk:
-            ref = po.attention_topk_f32(od, self.k_cfg, qh, kvh, tok_list=toks)
-            if isinstance(ref, tuple):
-                ref = ref[0]
-        else:
-            ref, _ = po.attention_f32(od, qh, kvh, tok_list=toks)
-        oracle_s = time.perf_counter() - t0
-        got = R.bf16_bits_to_f32(lay.out.cpu().numpy().view(np.uint16)).reshape(canvas, nq, lay.head_dim)
-        d = np.abs(got[toks] - ref[toks])
-        return {"max_abs": float(d.max()), "mean_abs": float(d.mean()), "finite": bool(np.isfinite(got).all()),
-                "oracle_s": oracle_s}

@@ -48,13 +48,14 @@ class Workload:
     def desc(self, **kw) -> capi.AttnDesc:
         dt = capi.DG_BF16 if self.dtype == "bf16" else capi.DG_F32
         flags = kw.pop("flags", 0)
+        default_partials = kw.pop("default_partials", False)   # leave the partial-row format to the library
         t_lo = 0
         if self.t_lo is not None:
             flags |= capi.DG_ATTN_F_T_LO_EXPLICIT
             t_lo = self.t_lo
         if self.sees_masked:
             flags |= capi.DG_ATTN_F_CAUSAL_SEES_MASKED
-        if not flags & capi.DG_ATTN_F_F32_PARTIALS:
+        if not default_partials and not flags & capi.DG_ATTN_F_F32_PARTIALS:
             # every generator below draws V from N(0, kv_std^2) (RMS-normalised or not): far inside the
             # f16 range, as are the V rows a model's cache holds after the producer's RMSNorm
             flags |= capi.DG_ATTN_F_F16_PARTIALS

@@ -52,3 +52,33 @@ def ref_kv_split(f):
     t = f.t_total()
     kv = np.asarray(f.kvcache, np.float32).reshape(t, 2, f.n_kv(), f.head_dim())
     return kv[:, 0], kv[:, 1]
+
+
+def schedule_oracle_check(sched, po, layer_index, toks):
+    """Layer `layer_index` of a diffgemma_amd.schedule.DenoiseSchedule: its output rows `toks` (and, for a
+    dense layer, their log-sum-exp) against the CPU oracle, on the inputs the device holds after the
+    producer ran (rotated q, cache with the canvas rows written)."""
+    import time
+    from diffgemma_amd import rounding as R
+    lay = sched.layers[layer_index]
+    canvas, nq = sched.canvas, sched.n_q_heads
+    qh = R.bf16_bits_to_f32(lay.q.cpu().numpy().view(np.uint16))
+    kvh = R.bf16_bits_to_f32(lay.cache.cpu().numpy().view(np.uint16))
+    od = po.make_desc(canvas, nq, lay.n_kv_heads, lay.head_dim, sched.kv_len, window=lay.window,
+                      kv_ring_mask=lay.ring_mask, layout="head_major", t_cap=lay.slots)
+    toks = np.asarray(toks, dtype=np.uint32)
+    t0 = time.perf_counter()
+    lse_rel = None
+    if lay.full and sched.global_topk:
+        ref = po.attention_topk_f32(od, sched.k_cfg, qh, kvh, tok_list=toks)
+        if isinstance(ref, tuple):
+            ref = ref[0]
+    else:
+        ref, ref_lse = po.attention_f32(od, qh, kvh, tok_list=toks)
+        got_lse = lay.lse.cpu().numpy().reshape(canvas, nq)
+        lse_rel = float(np.max(np.abs(got_lse[toks] - ref_lse[toks]) / np.abs(ref_lse[toks])))
+    oracle_s = time.perf_counter() - t0
+    got = R.bf16_bits_to_f32(lay.out.cpu().numpy().view(np.uint16)).reshape(canvas, nq, lay.head_dim)
+    d = np.abs(got[toks] - ref[toks])
+    return {"max_abs": float(d.max()), "mean_abs": float(d.mean()), "finite": bool(np.isfinite(got).all()),
+            "lse_rel": lse_rel, "oracle_s": oracle_s}

@@ -127,13 +127,13 @@ def test_model_full_fixture_midsize(gpu_ready, po):
 
 # ------------------------------------------------------------------ generic runner
 def run_workload(po, w, *, n_splits=0, kernel=capi.DG_KERNEL_AUTO, out_f32=False, toks=None, ring=None, flags=0,
-                 kv_override=None):
+                 kv_override=None, default_partials=False):
     import torch
     q, kv = W.generate(w)
     if kv_override is not None:
         kv = kv_override(kv)
     qd, kd = W.device_arrays(w, q, kv)
-    desc = w.desc(n_splits=n_splits, kernel=kernel, flags=flags)
+    desc = w.desc(n_splits=n_splits, kernel=kernel, flags=flags, default_partials=default_partials)
     if out_f32:
         desc.out_dtype = capi.DG_F32
     is_bf16_out = desc.out_dtype == capi.DG_BF16
@@ -154,14 +154,16 @@ def run_workload(po, w, *, n_splits=0, kernel=capi.DG_KERNEL_AUTO, out_f32=False
     return got[rows], got_lse[rows], ref[rows], ref_lse[rows]
 
 
-LSE_ABS = 2.0 ** -8
+LSE_ABS = 2.5e-3
 
 
-def check_tolerances(got, got_lse, ref, ref_lse, max_abs=MAX_ABS, mean_abs=MEAN_ABS):
-    """The benchmark tolerances on the output; the library's documented bound on the log-sum-exp,
-    |lse - exact| <= max(1e-3 |exact|, 2^-8): the row sum is taken over the probabilities as rounded
-    for the MFMA (the numbers P.V multiplies), which moves ln(sum) by up to 2^-8, so the relative
-    bound alone would fail rows whose LSE is small in magnitude.  Rows without a visible key: -inf."""
+def check_tolerances(got, got_lse, ref, ref_lse, max_abs=MAX_ABS, mean_abs=MEAN_ABS, strict_lse=False):
+    """The benchmark tolerances on the output.  Log-sum-exp: with strict_lse (the benchmark configurations)
+    the stated bound, 1e-3 relative, on every row; otherwise (arbitrary shapes and data) the library's
+    documented bound |lse - exact| <= max(1e-3 |exact|, 2.5e-3): the row sum is taken over the
+    probabilities as rounded for the MFMA (the numbers P.V multiplies), each within 2^-9 of its value, which
+    moves ln(sum) by up to 2^-9 = 1.95e-3, so the relative bound alone would fail rows whose LSE is small in
+    magnitude.  Rows without a visible key: -inf."""
     assert np.all(np.isfinite(got))
     assert max_abs_diff(got, ref) <= max_abs
     assert mean_abs_diff(got, ref) <= mean_abs
@@ -169,42 +171,56 @@ def check_tolerances(got, got_lse, ref, ref_lse, max_abs=MAX_ABS, mean_abs=MEAN_
     ok = np.isfinite(ref_lse)
     assert np.array_equal(np.isfinite(got_lse), ok)
     err = np.abs(got_lse[ok] - ref_lse[ok])
-    assert np.all(err <= np.maximum(LSE_REL * np.abs(ref_lse[ok]), LSE_ABS))
+    assert np.all(err <= np.maximum(LSE_REL * np.abs(ref_lse[ok]), 0.0 if strict_lse else LSE_ABS))
 
 
 # ------------------------------------------------------------------ benchmark configurations
 def test_cfg1_tiny_fp32(gpu_ready, po):
     """fp32 in, fp32 out; the library computes in f16 after a conversion pass."""
     got, lse, ref, ref_lse = run_workload(po, W.config("cfg1_tiny"))
-    check_tolerances(got, lse, ref, ref_lse, max_abs=2e-4, mean_abs=2e-5)
+    check_tolerances(got, lse, ref, ref_lse, max_abs=2e-4, mean_abs=2e-5, strict_lse=True)
 
 
 @pytest.mark.parametrize("name", ["cfg2_sliding", "cfg2_sliding_768"])
 def test_cfg2_sliding_window(gpu_ready, po, name):
-    check_tolerances(*run_workload(po, W.config(name)))
+    check_tolerances(*run_workload(po, W.config(name)), strict_lse=True)
 
 
 @pytest.mark.parametrize("name", ["cfg3_global", "cfg3_global_b", "cfg3_global_f16kv"])
 def test_cfg3_global_full_size(gpu_ready, po, name):
     """Full 32k-prefix shape, every row, mixed committed/bidirectional mask."""
-    check_tolerances(*run_workload(po, W.config(name)))
+    check_tolerances(*run_workload(po, W.config(name)), strict_lse=True)
+
+
+def test_cfg3_global_with_the_library_default_partial_rows(gpu_ready, po):
+    """The workload descriptors ask for f16 partial rows (DG_ATTN_F_F16_PARTIALS: the caller vouches for the
+    range of V in a bf16 cache).  Without the flag a bf16 cache gets fp32 partial rows: same tolerances, and the
+    two results differ by output roundings only."""
+    w = W.config("cfg3_global")
+    toks = np.arange(0, 256, 3, dtype=np.uint32)
+    f32p = run_workload(po, w, toks=toks, default_partials=True)
+    check_tolerances(*f32p, strict_lse=True)
+    f16p = run_workload(po, w, toks=toks)
+    diff = np.abs(f32p[0] - f16p[0])
+    assert diff.max() <= 2.0 ** -7 * max(1.0, np.abs(f32p[0]).max()) and np.mean(diff > 0) < 0.1
+    assert np.array_equal(f32p[1], f16p[1])
 
 
 def test_cfg3_unrounded_output_error_budget(gpu_ready, po):
     """fp32 output isolates the kernel's own error (bf16 probabilities) from output rounding."""
     toks = np.arange(0, 256, 5, dtype=np.uint32)
     got, lse, ref, ref_lse = run_workload(po, W.config("cfg3_global"), out_f32=True, toks=toks)
-    check_tolerances(got, lse, ref, ref_lse, max_abs=8e-3, mean_abs=3e-4)
+    check_tolerances(got, lse, ref, ref_lse, max_abs=8e-3, mean_abs=3e-4, strict_lse=True)
 
 
 def test_cfg4_long_context_rows(gpu_ready, po):
     """131072-key prefix with 1% of keys scaled x8 (peaked rows); oracle on a row sample."""
     toks = np.array([0, 1, 63, 64, 127, 128, 200, 255], dtype=np.uint32)
-    check_tolerances(*run_workload(po, W.config("cfg4_long"), toks=toks))
+    check_tolerances(*run_workload(po, W.config("cfg4_long"), toks=toks), strict_lse=True)
 
 
 def test_cfg5_sliding_layer_at_32k(gpu_ready, po):
-    check_tolerances(*run_workload(po, W.config("cfg5_sliding_32k")))
+    check_tolerances(*run_workload(po, W.config("cfg5_sliding_32k")), strict_lse=True)
 
 
 # ------------------------------------------------------------------ size-independent properties at full size
@@ -311,7 +327,7 @@ def test_dropped_weights_stay_below_rounding(gpu_ready, po):
     zero.  Rows built to make the most of that: one key at the top, half of the others 2^39 below it (kept),
     half 2^41 below (dropped) and carrying values a thousand times larger than the rest.  The result still
     meets the oracle far inside the tolerances (what is left is the bf16 rounding of the kept weights, which
-    moves ln(l) by up to 2^-8)."""
+    moves ln(l) by up to 2^-9)."""
     import torch
     w = W.Workload("drop", 64, 8, 2, 64, 4096 - 64, rms_norm=False, seed=5)
     q, kv = W.generate(w)

@@ -34,7 +34,8 @@ def test_dense_random_shape(gpu_ready, po, seed):
     toks = None if canvas * (kvl + canvas) * hq * hd < 6e9 else np.unique(np.linspace(0, canvas - 1, 24).round().astype(np.uint32))
     # (the two flags change which kernel instance runs, never the result: some seeds carry them)
     flags = (capi.DG_ATTN_F_KV_FROM_HBM if seed % 2 else 0) | (capi.DG_ATTN_F_STREAMED_MERGE if seed % 3 == 1 else 0)
-    check_tolerances(*run_workload(po, w, n_splits=splits, toks=toks, flags=flags))
+    # every third seed leaves the partial-row format to the library (fp32 for a bf16 cache) instead of asking for f16
+    check_tolerances(*run_workload(po, w, n_splits=splits, toks=toks, flags=flags, default_partials=seed % 3 == 2))
     if seed % 4 == 0:
         check_tolerances(*run_workload(po, w, kernel=capi.DG_KERNEL_SCALAR, toks=toks))
 

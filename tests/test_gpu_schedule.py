@@ -5,6 +5,8 @@ src/metal/step_kernel/runtime.rs:573-631, full layers src/metal/step_kernel/mod.
 import numpy as np
 import pytest
 
+from helpers import schedule_oracle_check
+
 pytestmark = pytest.mark.gpu
 
 N_ITER = 16
@@ -54,8 +56,9 @@ def test_replay_equals_eager_for_16_iterations_and_meets_the_oracle(sched, po):
             assert torch.equal(lay.out, want), (it, lay.index)
         if it in (0, N_ITER - 1):
             for idx in (0, 5, 29):
-                r = sched.oracle_check(po, idx, toks)
+                r = schedule_oracle_check(sched, po, idx, toks)
                 assert r["finite"] and r["max_abs"] <= 2e-2 and r["mean_abs"] <= 2e-3, (it, idx, r)
+                assert r["lse_rel"] <= 1e-3, (it, idx, r)      # per-row log-sum-exp, strictly relative
 
 
 def test_iterations_differ(sched):

@@ -230,3 +230,28 @@ def test_workload_table():
     assert w.t_lo == 2048 - 768
     with pytest.raises(KeyError):
         W.config("nope")
+
+
+def test_block_state_covers_every_block_partial():
+    """dg_attention_block_state_bytes must hold the carried state, a fresh state and the workspace of the
+    partial of ANY block [a, b) of the key range: the split count a range resolves to is not monotone in
+    its length, so a shorter block can need more partial rows than the whole range."""
+    lib = capi.load()
+    for hd, nkv in ((512, 2), (256, 8)):
+        L = capi.LayerOffsets()
+        L.head_dim, L.n_kv_heads, L.is_full, L.kv_ring_mask = hd, nkv, int(hd == 512), 0
+        dims = capi.AttnDims(256, 16, 0, 0)
+        for kv_len in list(range(0, 4200, 97)) + [1287, 32768, 131072]:
+            total, sb = C.c_size_t(0), C.c_size_t(0)
+            capi.check(lib.dg_attention_block_state_bytes(C.byref(L), C.byref(dims), kv_len, C.byref(total)))
+            d = A.make_desc(256, 16, nkv, hd, kv_len, q_dtype=capi.DG_BF16, kv_dtype=capi.DG_F16, out_dtype=capi.DG_BF16,
+                            flags=capi.DG_ATTN_F_OUT_TRUNCATE)
+            capi.check(lib.dg_attn_state_bytes(C.byref(d), C.byref(sb)))
+            state = (sb.value + 255) // 256 * 256
+            t_all = kv_len + 256
+            ends = sorted(set(list(range(32, t_all + 64, max(32, t_all // 61))) + [t_all, 1536]))
+            for b in ends:
+                for a in (0, b // 3 // 8 * 8):
+                    ws = C.c_size_t(0)
+                    capi.check(lib.dg_attn_partial_workspace_bytes(C.byref(d), a, b, C.byref(ws)))
+                    assert ws.value <= total.value - 2 * state, (hd, kv_len, a, b, ws.value, total.value, state)
