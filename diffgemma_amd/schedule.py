@@ -18,7 +18,7 @@ from typing import List, Optional
 
 import numpy as np
 
-from . import attention as A, attention_topk as T, capi, qk_rope_kv as QR, step_kv
+from . import attention as A, attention_topk as T, capi, qk_rope_kv as QR, rounding as R, step_kv
 
 
 @dataclass
