@@ -14,7 +14,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_NAME = "libdg_attn_hip.so"
 LIB_PATH = PKG_DIR / LIB_NAME
-SOURCES = ["dg_attn_api.hip", "attn_mfma.hip", "attn_aux.hip", "qk_rope_kv.hip", "attn_topk.hip", "kv_snapshot.hip"]
+SOURCES = ["dg_attn_api.hip", "attn_mfma.hip", "attn_wsplit.hip", "attn_aux.hip", "qk_rope_kv.hip", "attn_topk.hip", "kv_snapshot.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

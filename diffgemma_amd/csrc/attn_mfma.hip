@@ -63,62 +63,6 @@ template <bool F16>
 constexpr float kPOff = F16 ? 0.0f : 86.0f;
 constexpr float kDrop = 40.0f;
 
-// Score MFMAs, written as assembly so that their accumulator is an ordinary VGPR tuple.  O fills
-// all 256 accumulation registers at head_dim 512; the compiler gives every MFMA of such a
-// kernel an accumulation-register destination, which made it park one block of O in VGPRs
-// around each tile's score MFMAs (48 register moves per tile and wave).
-// The compiler does not know these are MFMAs, so the one hazard it would otherwise cover is
-// handled here: the last score MFMA of a tile (mfma_scores_last) is followed by the wait
-// states a non-MFMA read of the scores needs.  Back-to-back MFMAs that accumulate into the same registers need
-// no wait states, and operands that come from LDS are covered by the s_waitcnt the compiler
-// inserts for the asm operands.
-template <bool F16>
-__device__ __forceinline__ void mfma_scores_first(f32x16& s, u32x4 a, u32x4 b) {
-  if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
-  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
-}
-template <bool F16>
-__device__ __forceinline__ void mfma_scores_acc(f32x16& s, u32x4 a, u32x4 b) {
-  if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
-  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
-}
-// Last score MFMA of a tile, followed by 24 wait states: more than the 20 a 16-pass MFMA result
-// needs before a VALU may read it.  They are part of the same asm statement so that no
-// compiler-made register copy of the scores can land between the MFMA and the wait.
-template <bool F16>
-__device__ __forceinline__ void mfma_scores_last(f32x16& s, u32x4 a, u32x4 b) {
-  if constexpr (F16)
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
-  else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
-}
-
-// x *= c for values that live in accumulation registers, without the register allocator moving
-// them into the VGPR class.  Four at a time, so that no instruction waits for the one before it.
-__device__ __forceinline__ void scale_acc4(float& x0, float& x1, float& x2, float& x3, float c) {
-  float t0, t1, t2, t3;
-  asm volatile(
-      "v_accvgpr_read_b32 %4, %0\n\tv_accvgpr_read_b32 %5, %1\n\tv_accvgpr_read_b32 %6, %2\n\tv_accvgpr_read_b32 %7, %3\n\t"
-      "v_mul_f32 %4, %4, %8\n\tv_mul_f32 %5, %5, %8\n\tv_mul_f32 %6, %6, %8\n\tv_mul_f32 %7, %7, %8\n\t"
-      "v_accvgpr_write_b32 %0, %4\n\tv_accvgpr_write_b32 %1, %5\n\tv_accvgpr_write_b32 %2, %6\n\tv_accvgpr_write_b32 %3, %7\n\t"
-      "s_nop 3"   // the compiler does not see these writes: keep a following MFMA clear of them
-      : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
-      : "v"(c));
-}
-// Four values out of accumulation registers.  Spelled out so that the epilogue takes O from where
-// the tile loop left it, a few registers at a time: left to itself the compiler moves all of O
-// into VGPRs at the loop's exit, runs out of them and parks part of O in scratch memory, and the
-// reloads then queue behind the epilogue's own stores (one memory counter serves both), which
-// made every 32-row block wait for the previous block's stores to complete.
-template <bool FROM_ACC>
-__device__ __forceinline__ f32x4 acc_read4(const f32x16& a, int e) {
-  if constexpr (!FROM_ACC) return f32x4{a[e], a[e + 1], a[e + 2], a[e + 3]};   // smaller head_dim: O does not fill the registers
-  float t0, t1, t2, t3;
-  asm volatile("v_accvgpr_read_b32 %0, %4\n\tv_accvgpr_read_b32 %1, %5\n\tv_accvgpr_read_b32 %2, %6\n\tv_accvgpr_read_b32 %3, %7"
-               : "=v"(t0), "=v"(t1), "=v"(t2), "=v"(t3)
-               : "a"(a[e]), "a"(a[e + 1]), "a"(a[e + 2]), "a"(a[e + 3]));
-  return f32x4{t0, t1, t2, t3};
-}
 // dst = src for a score tile, as instructions the compiler cannot move or merge away; part I of
 // 8 copies elements 2 I and 2 I + 1
 template <int I>

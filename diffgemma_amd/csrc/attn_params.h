@@ -146,6 +146,7 @@ __device__ __forceinline__ void dbg_report(uint32_t* dbg, uint32_t code, uint32_
 // host-side launchers (defined next to their kernels)
 hipError_t launch_attn_scalar(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 hipError_t launch_attn_mfma(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
+hipError_t launch_attn_wsplit(const AttnParams& p, uint32_t head_dim, uint32_t kv_dtype, hipStream_t s);
 hipError_t launch_attn_merge(const AttnParams& p, uint32_t head_dim, bool streamed, hipStream_t s);
 hipError_t launch_state_merge(const StateMergeParams& p, hipStream_t s);
 // l[row] = 1 where m[row] is finite, else 0: completes a state whose rows are already normalised

@@ -16,6 +16,14 @@ namespace {
 
 using dg::kMaxSplits;
 constexpr size_t kAlign = 256;
+// most key tiles (of 32 keys) a row tile may see for the one-launch kernel to be chosen.  Step time in us,
+// one launch | split kernel + merge, 256-row canvas, 8 KV heads: head_dim 256: 40 tiles 19.8 | 23.4,
+// 72 tiles 28.5 | 27.5, 104 tiles 37.8 | 28.7; head_dim 128: 40 tiles 12.7 | 15.1, 72 tiles 18.9 | 19.3,
+// 104 tiles 25.0 | 21.4; head_dim 64: 40 tiles 11.6 | 13.4, 72 tiles 18.0 | 16.4.
+#ifndef DG_WSPLIT_MAX_TILES
+#define DG_WSPLIT_MAX_TILES 64
+#endif
+constexpr uint32_t kWsplitMaxTiles = DG_WSPLIT_MAX_TILES;
 
 inline size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
 inline uint32_t elem_size(uint32_t dt) { return dt == DG_F32 ? 4u : 2u; }
@@ -92,6 +100,7 @@ struct Plan {
   uint32_t e_dtype = DG_BF16;   // element type the kernels compute in (bf16 or f16)
   bool convert_q = false, gather_kv = false, q_is_bf16 = false;
   bool scalar = false;
+  bool wsplit = false;          // short key range, head_dim <= 256: keys split over the waves of a workgroup, one launch
   bool part_half = false;       // split partial rows travel as normalised f16 rows
   size_t off_q = 0, off_kv = 0, off_part_o = 0, off_part_ml = 0, total = 0;
   float scale = 1.0f;
@@ -185,8 +194,25 @@ int make_plan(const dg_attn_desc* d, int cus, Plan* pl, const uint32_t* key_rang
   pl->tile_end = std::max(pl->tile_first, (pl->clip_hi + dg::kBlockN - 1) / dg::kBlockN);
   const uint32_t ntiles = std::max(1u, pl->tile_end - pl->tile_first);
 
+  // A short key range at head_dim <= 256 (a sliding-window layer) runs as one launch in which the four waves
+  // of a workgroup split the keys and merge in LDS (attn_wsplit.hip): every workgroup then streams all keys
+  // its rows see, which pays while that is a few thousand keys.  The span is what one 32-row tile sees, not
+  // the union over the canvas (causal windowed rows each see window keys, the canvas window + canvas).
+  {
+    uint32_t span = 0;
+    if (d->causal_rows < d->canvas) span = std::max(span, pl->t_all - std::min(pl->lo_nc, pl->t_all));
+    if (d->causal_rows > 0) {
+      uint32_t c = d->kv_len + d->causal_rows;
+      if (d->window) c = std::min(c, d->window + dg::kBlockN);
+      if (d->flags & DG_ATTN_F_CAUSAL_SEES_MASKED) c = pl->t_all;
+      span = std::max(span, std::min(c, pl->t_all));
+    }
+    const uint32_t span_tiles = std::min(ntiles, span / dg::kBlockN + 2u);
+    pl->wsplit = !pl->scalar && hd <= 256 && d->n_splits == 0 && !(d->flags & DG_ATTN_F_SPLIT_OVER_WORKGROUPS) &&
+                 span_tiles <= kWsplitMaxTiles;
+  }
   uint32_t splits = d->n_splits;
-  if (pl->scalar) {
+  if (pl->scalar || pl->wsplit) {
     splits = 1;
   } else if (splits == 0) {
     // enough workgroups for every CU, but no split shorter than 6 tiles: below that the partial
@@ -414,7 +440,8 @@ int forward_planned(const dg_attn_desc* d, const Plan& pl, const void* q, const 
   }
   const bool prof = g_prof.active && 2 * (size_t)g_prof.used + 1 < g_prof.ev.size();
   if (prof) (void)hipEventRecord(g_prof.ev[2 * g_prof.used], s);
-  if (dg::launch_attn_mfma(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
+  if ((pl.wsplit ? dg::launch_attn_wsplit(p, hd, pl.e_dtype, s) : dg::launch_attn_mfma(p, hd, pl.e_dtype, s)) != hipSuccess)
+    return DG_ERR_LAUNCH;
   if (prof) {
     (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 1], s);
     ++g_prof.used;

@@ -88,6 +88,13 @@ typedef enum dg_kernel_sel {
                                               front (at most 8 splits, f16 partial rows, workspace below
                                               32 MiB).  Both give the same bits; the flag is there to compare them. */
 
+#define DG_ATTN_F_SPLIT_OVER_WORKGROUPS 0x80u /* head_dim <= 256 and a short key range (a sliding-window layer): the
+                                              library runs one launch in which the waves of a workgroup split the
+                                              keys and merge in LDS.  This flag asks for the general kernel instead
+                                              (keys split over workgroups, partial rows in the workspace, a merge
+                                              launch), as does an explicit n_splits.  Results agree to the rounding
+                                              of the probabilities; the flag is there to compare the two. */
+
 typedef struct dg_attn_desc {
   uint32_t canvas;        /* query rows; the reference passes active_canvas (256/128/64) */
   uint32_t n_q_heads;
@@ -129,8 +136,9 @@ int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits);
  * log-sum-exp of the scaled scores (NULL to skip; a row with no visible key gets -inf and
  * an all-zero output row).  Accuracy of lse: the row sum is taken over the probabilities as
  * rounded to the MFMA operand type (the numbers P.V multiplies, so that out is an exact
- * weighted mean): each is within 2^-9 of its value (bf16; 2^-12 with an f16 cache), which moves
- * ln(sum) by at most 2^-9 = 1.95e-3 absolute: |lse - exact| <= max(1e-3 |exact|, 2.5e-3). */
+ * weighted mean): bf16 keeps 8 significant bits, so each is within 2^-8 of its value (2^-11 with an f16
+ * cache), and on a row with one dominant key nothing averages out: ln(sum) moves by at most 2^-8 = 3.9e-3
+ * absolute: |lse - exact| <= max(1e-3 |exact|, 2^-8). */
 int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
                     void* workspace, size_t workspace_bytes, void* stream);
 

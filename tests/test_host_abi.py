@@ -136,8 +136,16 @@ def test_layout_helpers():
 def test_split_planning():
     assert capi.resolved_splits(W.config("cfg3_global").desc()) == 8          # 32 (tile, head) pairs x 8 = 256 workgroups
     assert capi.resolved_splits(W.config("cfg4_long").desc()) == 8
-    assert capi.resolved_splits(W.config("cfg2_sliding").desc()) == 6            # 40 visible tiles, 7 to a split (none shorter than 6)
-    assert capi.resolved_splits(W.config("cfg2_sliding_768").desc()) == 5        # 32 visible tiles, 7 to a split
+    # a sliding layer (head_dim 256, 40 visible key tiles) runs as one launch, keys split over the waves of a
+    # workgroup: no splits over workgroups, no workspace; asked for the general kernel it takes 6 splits
+    assert capi.resolved_splits(W.config("cfg2_sliding").desc()) == 1
+    assert capi.workspace_bytes(W.config("cfg2_sliding").desc()) == 0
+    over_wg = capi.DG_ATTN_F_SPLIT_OVER_WORKGROUPS
+    assert capi.resolved_splits(W.config("cfg2_sliding").desc(flags=over_wg)) == 6        # 40 visible tiles, 7 to a split (none shorter than 6)
+    assert capi.resolved_splits(W.config("cfg2_sliding_768").desc(flags=over_wg)) == 5    # 32 visible tiles, 7 to a split
+    assert capi.workspace_bytes(W.config("cfg2_sliding").desc(flags=over_wg)) == 6 * 8 * 512 * (256 * 2 + 2 * 4)
+    # the same head_dim over a long unwindowed range goes to the general kernel by itself
+    assert capi.resolved_splits(A.make_desc(256, 16, 8, 256, 8192)) == 8
     assert capi.resolved_splits(A.make_desc(2, 4, 2, 32, 2)) == 1                 # one tile: nothing to split
     assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, n_splits=3)) == 3
     assert capi.resolved_splits(A.make_desc(256, 16, 2, 512, 32768, kernel=capi.DG_KERNEL_SCALAR)) == 1
