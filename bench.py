@@ -226,6 +226,21 @@ def bench_schedule(args):
     torch.cuda.synchronize()
     block_ms = (time.perf_counter() - t0) * 1e3
 
+    # what following the committed prefix costs: recording the graph again for the new kv_len (what launches with a
+    # baked-in kv_len need after every committed block) against rewriting the one device word the *_dev entry points
+    # read (diffgemma_amd.schedule with kv_len_max set; tests/test_gpu_schedule.py replays one graph at two prefixes)
+    t0 = time.perf_counter()
+    sc.capture()
+    sc.replay()
+    torch.cuda.synchronize()
+    recapture_ms = (time.perf_counter() - t0) * 1e3
+    word = torch.zeros(12, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    word[0] = kv_len + canvas
+    torch.cuda.synchronize()
+    device_word_ms = (time.perf_counter() - t0) * 1e3
+
     flops_iter = sc.flops_per_iteration
     achieved = flops_iter / (ms * 1e-3) / 1e12
     res = {"metric": "denoise attention, 30-layer stack (25 sliding + 5 global) @ 32k prefix: TFLOP/s of producer + "
@@ -243,6 +258,7 @@ def bench_schedule(args):
            "denoise_block": {"iterations": n_block, "end_to_end_ms": block_ms,
                              "canvas_tokens_per_s": canvas / (block_ms / n_block * 1e-3)},
            "settle": {"replays": n_settle},
+           "prefix_advance": {"record_graph_again_ms": recapture_ms, "rewrite_device_kv_len_ms": device_word_ms},
            "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                         "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
                         "kernel": "whole iteration: 30 x (qk_rope_kv_kernel, attn_mfma_kernel, attn_merge_kernel)",

@@ -194,6 +194,23 @@ def forward(desc: capi.AttnDesc, q, kv, out, lse=None, workspace=None) -> None:
                                    lse.data_ptr() if lse is not None else None, ws_ptr, ws_bytes, stream_handle()))
 
 
+def forward_dev(desc: capi.AttnDesc, step_dev, q, kv, out, lse=None, workspace=None) -> None:
+    """dg_attn_forward_dev: kv_len is read from the device StepParams `step_dev` (an int32 tensor of 12 words,
+    kv_len first) when the kernels run; desc.kv_len is the largest prefix planned for."""
+    lib = capi.load()
+    ws_ptr, ws_bytes = (workspace.data_ptr(), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
+    capi.check(lib.dg_attn_forward_dev(C.byref(desc), step_dev.data_ptr(), q.data_ptr(), kv.data_ptr(), out.data_ptr(),
+                                       lse.data_ptr() if lse is not None else None, ws_ptr, ws_bytes, stream_handle()))
+
+
+def device_step_params(kv_len: int, kv_write_end: int = 0xFFFFFFFF):
+    """A device copy of the reference's StepParams (12 words; kv_len is word 0, kv_write_end word 11)."""
+    torch = _torch()
+    host = np.zeros(12, dtype=np.uint32)
+    host[0], host[11] = kv_len, kv_write_end
+    return torch.from_numpy(host.view(np.int32)).cuda()
+
+
 def state_bytes(desc: capi.AttnDesc) -> int:
     n = C.c_size_t(0)
     capi.check(capi.load().dg_attn_state_bytes(C.byref(desc), C.byref(n)))

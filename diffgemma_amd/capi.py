@@ -46,6 +46,7 @@ EXPORTS = (
     "dg_attn_forward_static", "dg_attn_static_scratch_bytes",
     "dg_attn_state_bytes", "dg_attn_partial_workspace_bytes", "dg_attn_partial", "dg_attn_merge",
     "dg_attention_dispatch_block", "dg_attention_block_state_bytes",
+    "dg_attn_forward_dev", "dg_attention_dispatch_dev", "dg_qk_rope_kv_dev", "dg_qk_rope_kv_dispatch_dev",
 )
 
 
@@ -147,6 +148,15 @@ def load():
     lib.dg_attn_resolved_splits.restype = C.c_int
     lib.dg_attn_forward.argtypes = [P(AttnDesc), VP, VP, VP, VP, VP, C.c_size_t, VP]
     lib.dg_attn_forward.restype = C.c_int
+    lib.dg_attn_forward_dev.argtypes = [P(AttnDesc), VP, VP, VP, VP, VP, VP, C.c_size_t, VP]
+    lib.dg_attn_forward_dev.restype = C.c_int
+    lib.dg_attention_dispatch_dev.argtypes = [VP, VP, VP, P(LayerOffsets), VP, C.c_uint32, P(AttnDims), VP, VP,
+                                              C.c_size_t, VP]
+    lib.dg_attention_dispatch_dev.restype = C.c_int
+    lib.dg_qk_rope_kv_dev.argtypes = [P(RopeDesc), VP, VP, VP, VP, VP, VP, VP, VP, VP]
+    lib.dg_qk_rope_kv_dev.restype = C.c_int
+    lib.dg_qk_rope_kv_dispatch_dev.argtypes = [VP, VP, VP, VP, VP, P(LayerOffsets), VP, P(AttnDims), VP, VP]
+    lib.dg_qk_rope_kv_dispatch_dev.restype = C.c_int
     lib.dg_attn_forward_static.argtypes = [P(AttnDesc), VP, VP, VP, VP, VP]
     lib.dg_attn_forward_static.restype = C.c_int
     lib.dg_attn_static_scratch_bytes.argtypes = []

@@ -103,7 +103,8 @@ __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
 }
 
 template <int D, bool F16, bool TOUCH>
-__global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p_in) {
+  const AttnParams p = resolve_step(p_in);
   using L = Lay<D>;
   constexpr int NSTEP = D / 16, NDB = D / 32;
   // P.V work split: DSPLIT groups of d-blocks x RSPLIT groups of row-blocks = 4 waves

@@ -26,6 +26,9 @@ struct AttnParams {
                        // index space in f16 holding accumulators divided by the split's row sum
   float* part_ml;      // [split][hkv][rows_pad][2] (m in log2 units, l)
   uint32_t* dbg;       // 4 words, first-writer-wins, or null
+  const uint32_t* step_dev;   // device copy of the reference's StepParams, or null: when set, kv_len is read from its
+                              // first word when the kernel runs (resolve_step) and the kv_len below is the largest
+                              // prefix the launch was planned for
   int64_t k_tok_stride, k_head_stride, v_tok_stride, v_head_stride;  // elements
   uint32_t canvas, hq, hkv, group;
   uint32_t kv_len, t_all;
@@ -41,6 +44,8 @@ struct AttnParams {
   uint32_t out_dtype, out_trunc;
   uint32_t part_half;    // split partials are normalised f16 rows instead of unnormalised fp32 ones
   uint32_t touch_ahead;  // head_dim 512: touch key/value tiles into the L2 some tiles before they are loaded
+  uint32_t lo_explicit;  // lo_nc was given by the caller (not the window rule)
+  uint32_t sees_masked;  // causal rows also see the canvas keys behind the causal rows
   float scale_log2;      // softmax_scale * log2(e)
 };
 
@@ -73,6 +78,32 @@ struct StateMergeParams {
   uint32_t out_dtype, out_trunc;
   uint32_t* dbg;
 };
+
+// The reference binds StepParams as a device buffer (src/metal/step_kernel/enc.rs:2177-2220, buffer 4), so the
+// prefix length a recorded command sequence works on is read when it runs.  With step_dev set, the same here:
+// kv_len comes from device memory (clamped to the prefix the launch was planned for: grid, split count and
+// workspace follow that maximum) and everything derived from it is worked out again, the way the host does it
+// in make_plan.  The key range is the whole one (a key-range partial takes kv_len from the host).
+__device__ __forceinline__ AttnParams resolve_step(const AttnParams& in) {
+  AttnParams p = in;
+  if (in.step_dev == nullptr) return p;
+  const uint32_t kv = (uint32_t)__builtin_amdgcn_readfirstlane((int)min(in.step_dev[0], in.kv_len));
+  p.kv_len = kv;
+  p.t_all = kv + p.canvas;
+  const bool windowed = p.win_m1 != 0xffffffffu;
+  if (!p.lo_explicit) p.lo_nc = (windowed && kv > p.win_m1) ? kv - p.win_m1 : 0u;
+  p.lo_nc = min(p.lo_nc, p.t_all);
+  p.extra_lo = p.sees_masked ? min(kv + p.causal_rows, p.t_all) : p.t_all;
+  uint32_t lo_all = 0xffffffffu;
+  if (p.causal_rows < p.canvas) lo_all = min(lo_all, p.lo_nc);
+  if (p.causal_rows > 0u) lo_all = min(lo_all, (windowed && kv > p.win_m1) ? kv - p.win_m1 : 0u);
+  lo_all = min(lo_all, p.t_all);
+  p.t_clip_lo = 0u;
+  p.t_clip_hi = p.t_all;
+  p.tile_first = lo_all / (uint32_t)kBlockN;
+  p.tile_end = max(p.tile_first, (p.t_all + (uint32_t)kBlockN - 1u) / (uint32_t)kBlockN);
+  return p;
+}
 
 struct RowBounds {
   uint32_t lo, hi, extra;  // visible iff (lo <= t < hi) or (extra <= t), and t < t_all

@@ -80,7 +80,8 @@ __device__ __forceinline__ void ws_issue_tile(const TileLoad& tl, uint32_t lane)
 }
 
 template <int D, bool F16>
-__global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in) {
+  const AttnParams p = resolve_step(p_in);
   using L = Lay<D>;
   static_assert(!L::PAD, "head_dim 512 does not fit: O alone would fill the register file");
   constexpr int NSTEP = D / 16, NDB = D / 32, NBLK = L::NBLK;

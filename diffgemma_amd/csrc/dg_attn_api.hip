@@ -403,6 +403,8 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   p.out_dtype = d->out_dtype;
   p.out_trunc = (d->flags & DG_ATTN_F_OUT_TRUNCATE) ? 1u : 0u;
   p.part_half = pl.part_half ? 1u : 0u;
+  p.lo_explicit = (d->flags & DG_ATTN_F_T_LO_EXPLICIT) ? 1u : 0u;
+  p.sees_masked = (d->flags & DG_ATTN_F_CAUSAL_SEES_MASKED) ? 1u : 0u;
   // key/value rows this call streams: more than the 256 MiB memory-side cache holds cannot have
   // stayed there from the previous call, whatever else runs in between (131072 keys: 0.933 -> 0.912 ms)
   const uint64_t kv_streamed = 2ull * d->n_kv_heads * (uint64_t)(pl.tile_end - pl.tile_first) * dg::kBlockN * d->head_dim * 2ull;
@@ -416,7 +418,7 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
 namespace {
 // One attention call with its plan made: validation of the pointers, parameter block, launches.
 int forward_planned(const dg_attn_desc* d, const Plan& pl, const void* q, const void* kv_base, void* out, float* lse,
-                    void* workspace, size_t workspace_bytes, void* stream) {
+                    void* workspace, size_t workspace_bytes, void* stream, const uint32_t* step_dev = nullptr) {
   int rc = DG_OK;
   if (pl.total > 0 && (!workspace || workspace_bytes < pl.total)) return DG_ERR_WORKSPACE;
   if (pl.total > 0 && ((uintptr_t)workspace % 16) != 0) return DG_ERR_WORKSPACE;
@@ -433,6 +435,8 @@ int forward_planned(const dg_attn_desc* d, const Plan& pl, const void* q, const 
     p.part_ml = (float*)(ws + pl.off_part_ml);
   }
   p.dbg = g_tls_dbg;  // set only while dg_attention_dispatch is on the stack
+  p.step_dev = step_dev;
+  if (step_dev && (pl.scalar || pl.gather_kv)) return DG_ERR_UNSUPPORTED;   // (the f32 cache copy is made for a host-known length)
 
   if (pl.scalar) {
     if (dg::launch_attn_scalar(p, hd, pl.e_dtype, s) != hipSuccess) return DG_ERR_LAUNCH;
@@ -461,6 +465,19 @@ int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, v
   rc = make_plan(d, di.cus, &pl);
   if (rc != DG_OK) return rc;
   return forward_planned(d, pl, q, kv_base, out, lse, workspace, workspace_bytes, stream);
+}
+
+int dg_attn_forward_dev(const dg_attn_desc* d, const dg_step_params* step_dev, const void* q, const void* kv_base, void* out,
+                        float* lse, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d || !step_dev || !q || !kv_base || !out) return DG_ERR_NULL;
+  if (((uintptr_t)step_dev % 4) != 0) return DG_ERR_LAYOUT;
+  DeviceInfo di;
+  int rc = device_info(&di);
+  if (rc != DG_OK) return rc;
+  Plan pl;
+  rc = make_plan(d, di.cus, &pl);
+  if (rc != DG_OK) return rc;
+  return forward_planned(d, pl, q, kv_base, out, lse, workspace, workspace_bytes, stream, (const uint32_t*)step_dev);
 }
 
 size_t dg_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
@@ -708,6 +725,18 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
   desc_from_reference(L, dims, P->kv_len, &d);
   g_tls_dbg = (uint32_t*)dbg;
   const int rc = dg_attn_forward(&d, q, kvcache, out, nullptr, attn_state, attn_state_bytes, stream);
+  g_tls_dbg = nullptr;
+  return rc;
+}
+
+int dg_attention_dispatch_dev(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                              const dg_step_params* P_dev, uint32_t kv_len_max, const dg_attn_dims* dims,
+                              dg_debug_status* dbg, void* attn_state, size_t attn_state_bytes, void* stream) {
+  if (!L || !P_dev || !dims) return DG_ERR_NULL;
+  dg_attn_desc d;
+  desc_from_reference(L, dims, kv_len_max, &d);
+  g_tls_dbg = (uint32_t*)dbg;
+  const int rc = dg_attn_forward_dev(&d, P_dev, q, kvcache, out, nullptr, attn_state, attn_state_bytes, stream);
   g_tls_dbg = nullptr;
   return rc;
 }

@@ -28,6 +28,8 @@ struct RopeParams {
   const uint16_t* qw;    // [hd] bf16 norm weights
   const uint16_t* kw;
   uint32_t* dbg;
+  const uint32_t* step_dev;   // device copy of the reference's StepParams, or null: kv_len (word 0) and kv_write_end
+                              // (word 11) are then read from it when the kernel runs
   int64_t k_tok_stride, k_head_stride, v_tok_stride, v_head_stride;  // elements
   uint32_t canvas, hq, hkv, hd;
   uint32_t kv_len, kv_write_end, ring_mask;
@@ -111,8 +113,11 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   const uint32_t hd = p.hd;
   const bool is_q = h < p.hq, is_k = !is_q && h < p.hq + p.hkv;
   const uint32_t hh = is_q ? h : (h - p.hq) % p.hkv;
-  const uint32_t pos = p.kv_len + tok;
-  const bool kv_write = pos < p.kv_write_end;
+  // (the reference binds StepParams as a device buffer, qk_rope_kv.metal:30-38: read at execution time)
+  const uint32_t kv_len = p.step_dev ? (uint32_t)__builtin_amdgcn_readfirstlane((int)p.step_dev[0]) : p.kv_len;
+  const uint32_t kv_write_end = p.step_dev ? (uint32_t)__builtin_amdgcn_readfirstlane((int)p.step_dev[11]) : p.kv_write_end;
+  const uint32_t pos = kv_len + tok;
+  const bool kv_write = pos < kv_write_end;
   const int64_t slot = p.ring_mask ? (pos & p.ring_mask) : pos;
 
   uint16_t* row_inplace = is_q ? p.q + ((size_t)tok * p.hq + hh) * hd : p.k + ((size_t)tok * p.hkv + hh) * hd;
@@ -194,9 +199,10 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
 
 extern "C" {
 
-int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* kv_base, const void* q_norm_w,
-                  const void* k_norm_w, dg_debug_status* dbg, void* stream) {
+static int rope_launch(const dg_rope_desc* d, const dg_step_params* step_dev, void* q, void* k, const void* v, void* kv_base,
+                       const void* q_norm_w, const void* k_norm_w, dg_debug_status* dbg, void* stream) {
   if (!d || !q || !k || !kv_base || !q_norm_w || !k_norm_w) return DG_ERR_NULL;
+  if (((uintptr_t)step_dev % 4) != 0) return DG_ERR_LAYOUT;
   if (!d->v_from_k && !v) return DG_ERR_NULL;
   const uint32_t hd = d->head_dim;
   if (!(hd == 32 || hd == 64 || hd == 128 || hd == 256 || hd == 512)) return DG_ERR_SHAPE;
@@ -218,6 +224,7 @@ int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* 
   p.qw = (const uint16_t*)q_norm_w;
   p.kw = (const uint16_t*)k_norm_w;
   p.dbg = (uint32_t*)dbg;
+  p.step_dev = (const uint32_t*)step_dev;
   p.k_tok_stride = d->k_tok_stride;
   p.k_head_stride = d->k_head_stride;
   p.v_tok_stride = d->v_tok_stride;
@@ -255,16 +262,28 @@ int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* 
   return hipGetLastError() == hipSuccess ? DG_OK : DG_ERR_LAUNCH;
 }
 
-int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
-                           const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream) {
-  if (!L || !P || !dims || !blob) return DG_ERR_NULL;
+int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* kv_base, const void* q_norm_w,
+                  const void* k_norm_w, dg_debug_status* dbg, void* stream) {
+  return rope_launch(d, nullptr, q, k, v, kv_base, q_norm_w, k_norm_w, dbg, stream);
+}
+
+int dg_qk_rope_kv_dev(const dg_rope_desc* d, const dg_step_params* step_dev, void* q, void* k, const void* v, void* kv_base,
+                      const void* q_norm_w, const void* k_norm_w, dg_debug_status* dbg, void* stream) {
+  if (!step_dev) return DG_ERR_NULL;
+  return rope_launch(d, step_dev, q, k, v, kv_base, q_norm_w, k_norm_w, dbg, stream);
+}
+
+// The reference's argument block -> descriptor; kv_len / kv_write_end from the host copy of P, or (P == null) left to
+// the device copy.
+static void rope_desc_from_reference(const dg_layer_offsets* L, const dg_step_params* P, const dg_attn_dims* dims,
+                                     dg_rope_desc* out) {
   dg_rope_desc d{};
   d.canvas = dims->canvas;
   d.n_q_heads = dims->n_q_heads;
   d.n_kv_heads = L->n_kv_heads;
   d.head_dim = L->head_dim;
-  d.kv_len = P->kv_len;
-  d.kv_write_end = P->kv_write_end;
+  d.kv_len = P ? P->kv_len : 0u;
+  d.kv_write_end = P ? P->kv_write_end : 0xffffffffu;
   d.kv_ring_mask = L->kv_ring_mask;
   d.is_full = L->is_full;
   d.v_from_k = L->v_proj == 0 ? 1u : 0u;
@@ -277,7 +296,24 @@ int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void*
   d.v_base_off = row;
   d.v_tok_stride = 2 * row;
   d.v_head_stride = L->head_dim;
+  *out = d;
+}
+
+int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
+                           const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream) {
+  if (!L || !P || !dims || !blob) return DG_ERR_NULL;
+  dg_rope_desc d;
+  rope_desc_from_reference(L, P, dims, &d);
   return dg_qk_rope_kv(&d, q, k, v, kvcache, (const char*)blob + L->q_norm, (const char*)blob + L->k_norm, dbg, stream);
+}
+
+int dg_qk_rope_kv_dispatch_dev(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
+                               const dg_step_params* P_dev, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream) {
+  if (!L || !P_dev || !dims || !blob) return DG_ERR_NULL;
+  dg_rope_desc d;
+  rope_desc_from_reference(L, nullptr, dims, &d);
+  return dg_qk_rope_kv_dev(&d, P_dev, q, k, v, kvcache, (const char*)blob + L->q_norm, (const char*)blob + L->k_norm, dbg,
+                           stream);
 }
 
 }  // extern "C"

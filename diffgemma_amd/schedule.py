@@ -50,6 +50,9 @@ class DenoiseSchedule:
     canvas: int = 256
     n_q_heads: int = 16
     kv_len: int = 32768
+    kv_len_max: Optional[int] = None   # set: the committed prefix lives in device memory (a device StepParams the
+                                       # kernels read when they run, as the reference binds it, enc.rs:2177-2220) and
+                                       # may be advanced up to this value between replays of ONE recorded graph
     ring: int = 2048
     window: int = 1024
     n_layers: int = step_kv.N_LAYERS
@@ -60,6 +63,7 @@ class DenoiseSchedule:
     flops_per_iteration: float = 0.0
     graph: Optional[object] = None
     topk_ws: Optional[object] = None
+    step_dev: Optional[object] = None   # device StepParams (int32 x 12) when kv_len_max is set
     k_cfg: Optional[object] = None
 
     def build(self) -> "DenoiseSchedule":
@@ -74,7 +78,10 @@ class DenoiseSchedule:
             x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
             return x.to(torch.bfloat16).view(torch.int16).reshape(-1)
 
-        canvas, nq, kv_len = self.canvas, self.n_q_heads, self.kv_len
+        canvas, nq = self.canvas, self.n_q_heads
+        kv_len = self.kv_len_max if self.kv_len_max is not None else self.kv_len   # what the layers are planned for
+        assert self.kv_len <= kv_len
+        self.step_dev = A.device_step_params(self.kv_len) if self.kv_len_max is not None else None
         for i in range(self.n_layers):
             full = i in self.full_layers
             hd, nkv = (512, 2) if full else (256, 8)
@@ -110,6 +117,12 @@ class DenoiseSchedule:
             self.flops_per_iteration += lay.flops
         return self
 
+    def set_kv_len(self, kv_len: int) -> None:
+        """A block was committed: the prefix grows.  Only the device word changes; a recorded graph stays valid."""
+        assert self.step_dev is not None and kv_len <= self.kv_len_max
+        self.kv_len = kv_len
+        self.step_dev[0] = kv_len
+
     def regenerate(self, iteration: int) -> None:
         """Canvas projections of iteration `iteration`: N(0, 1) from the device generator keyed by seed + iteration."""
         import torch
@@ -122,6 +135,12 @@ class DenoiseSchedule:
         """Enqueue one iteration on the current stream: per layer the producer, then attention."""
         st = A.stream_handle()
         for lay in self.layers:
+            if self.step_dev is not None:
+                capi.check(self._lib.dg_qk_rope_kv_dev(C.byref(lay.rope_desc), self.step_dev.data_ptr(), lay.q.data_ptr(),
+                                                       lay.k.data_ptr(), lay.v.data_ptr(), lay.cache.data_ptr(),
+                                                       lay.q_norm_w.data_ptr(), lay.k_norm_w.data_ptr(), None, st))
+                A.forward_dev(lay.attn_desc, self.step_dev, lay.q, lay.cache, lay.out, lay.lse, lay.workspace)
+                continue
             capi.check(self._lib.dg_qk_rope_kv(C.byref(lay.rope_desc), lay.q.data_ptr(), lay.k.data_ptr(),
                                                lay.v.data_ptr(), lay.cache.data_ptr(), lay.q_norm_w.data_ptr(),
                                                lay.k_norm_w.data_ptr(), None, st))

@@ -47,6 +47,8 @@ typedef enum dg_status {
   DG_ERR_SCRATCH_LIMIT = -10 /* dg_attn_forward_static: the call needs more scratch than the library holds */
 } dg_status;
 
+struct dg_step_params;   /* below */
+
 typedef enum dg_dtype { DG_BF16 = 0, DG_F16 = 1, DG_F32 = 2 } dg_dtype;
 
 typedef enum dg_kernel_sel {
@@ -141,6 +143,18 @@ int dg_attn_resolved_splits(const dg_attn_desc* d, uint32_t* out_splits);
  * absolute: |lse - exact| <= max(1e-3 |exact|, 2^-8). */
 int dg_attn_forward(const dg_attn_desc* d, const void* q, const void* kv_base, void* out, float* lse,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* dg_attn_forward with the prefix length read on the device when the kernels run, the way the reference binds
+ * StepParams as a device buffer (src/metal/step_kernel/enc.rs:2177-2220, buffer 4: its kernels read kv_len at
+ * execution time, so one encoded step serves every committed prefix).  step_dev is a DEVICE dg_step_params (only
+ * kv_len is read); d->kv_len is the largest prefix the call has to cover: grid, split count and workspace are planned
+ * for it (dg_attn_workspace_bytes with the same descriptor), and a device value above it is clamped to it.  A HIP
+ * graph recorded with this entry stays valid while the caller advances kv_len in device memory after every committed
+ * block (src/metal/step_generate/turn.rs:575-660) instead of recording again.  For every device value the result is
+ * that of dg_attn_forward with kv_len set to it, bit for bit when both resolve to the same split count.  Not for the
+ * scalar cross-check kernel or an f32 cache (DG_ERR_UNSUPPORTED). */
+int dg_attn_forward_dev(const dg_attn_desc* d, const struct dg_step_params* step_dev, const void* q, const void* kv_base,
+                        void* out, float* lse, void* workspace, size_t workspace_bytes, void* stream);
 
 /* dg_attn_forward for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): no workspace argument.  It has no
@@ -260,6 +274,13 @@ int dg_attention_dispatch(const void* q, const void* kvcache, void* out, const d
 int dg_attention_state_bytes(const dg_layer_offsets* L, const dg_attn_dims* dims, uint32_t kv_len,
                              size_t* out_bytes);
 
+/* dg_attention_dispatch with P bound as the reference binds it: a DEVICE dg_step_params whose kv_len is read when the
+ * kernels run.  kv_len_max (host) is the largest prefix the session can reach; attn_state is sized with it
+ * (dg_attention_state_bytes(L, dims, kv_len_max)). */
+int dg_attention_dispatch_dev(const void* q, const void* kvcache, void* out, const dg_layer_offsets* L,
+                              const dg_step_params* P_dev, uint32_t kv_len_max, const dg_attn_dims* dims,
+                              dg_debug_status* dbg, void* attn_state, size_t attn_state_bytes, void* stream);
+
 /* dg_attention_dispatch for one block of keys, the way the reference's host loop dispatches
  * attention_mma_full (enc.rs:2261-2291: blocks in order, blk = {t_begin, t_end, is_first, is_last}
  * bound at index 7): the first block starts the state in attn_state, a middle block folds its keys
@@ -339,12 +360,22 @@ typedef struct dg_rope_desc {
 int dg_qk_rope_kv(const dg_rope_desc* d, void* q, void* k, const void* v, void* kv_base, const void* q_norm_w,
                   const void* k_norm_w, dg_debug_status* dbg, void* stream);
 
+/* dg_qk_rope_kv with kv_len and kv_write_end read from a DEVICE dg_step_params when the kernel runs (the reference
+ * binds StepParams as a device buffer, qk_rope_kv.metal:30-38); d->kv_len and d->kv_write_end are ignored.  Pairs
+ * with dg_attn_forward_dev: a recorded producer + attention sequence follows the committed prefix without being
+ * recorded again.  The cache must have room for the largest prefix + canvas the caller will set. */
+int dg_qk_rope_kv_dev(const dg_rope_desc* d, const struct dg_step_params* step_dev, void* q, void* k, const void* v,
+                      void* kv_base, const void* q_norm_w, const void* k_norm_w, dg_debug_status* dbg, void* stream);
+
 /* The same with exactly the buffers the reference kernel binds (qk_rope_kv.metal:30-38): q, k, v
  * in the arena, the whole f16 KV buffer (the kernel adds L->kv_region), the weight blob (norm
  * weights at L->q_norm / L->k_norm, bf16), host copies of L / P / dims.  q and k are stored with
  * the reference's truncating bf16 store, the cache as f16 (kv_store). */
 int dg_qk_rope_kv_dispatch(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
                            const dg_step_params* P, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream);
+/* ... with P bound as a device buffer, as the reference binds it */
+int dg_qk_rope_kv_dispatch_dev(void* q, void* k, void* v, void* kvcache, const void* blob, const dg_layer_offsets* L,
+                               const dg_step_params* P_dev, const dg_attn_dims* dims, dg_debug_status* dbg, void* stream);
 
 /* ---- KV-cache layout arithmetic (host) ---- */
 uint64_t dg_kv_row_bytes(uint32_t head_dim, uint32_t kv_dtype);

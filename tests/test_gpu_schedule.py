@@ -77,3 +77,50 @@ def test_iterations_differ(sched):
     sched.replay()
     torch.cuda.synchronize()
     assert not torch.equal(a, sched.layers[5].out)
+
+
+def test_one_recorded_graph_follows_the_committed_prefix(gpu_ready, po):
+    """The reference binds StepParams as a device buffer (src/metal/step_kernel/enc.rs:2177-2220), so the step it
+    encoded serves every committed prefix (src/metal/step_generate/turn.rs:575-660: kv_len += 256 per committed
+    block).  Same here with the *_dev entry points: one graph recorded at prefix 32768, replayed there and, after
+    only the device word changed, at 33024.  At both lengths the replay equals plain launches bit for bit and
+    meets the oracle; at the first it also equals the graph-free schedule that bakes kv_len into its launches."""
+    import torch
+    from diffgemma_amd import schedule
+    kv0, kv1 = 32768, 33024
+    sc = schedule.DenoiseSchedule(kv_len=kv0, kv_len_max=kv1).build()
+    plain = schedule.DenoiseSchedule(kv_len=kv0).build()
+    for a, b in zip(sc.layers, plain.layers):      # the same cache rows behind both (they are drawn per layer size)
+        src = a.cache.view(2, a.n_kv_heads, a.slots, a.head_dim)
+        b.cache.view(2, b.n_kv_heads, b.slots, b.head_dim).copy_(src[:, :, :b.slots])
+    sc.regenerate(0)
+    sc.run_eager()
+    torch.cuda.synchronize()
+    sc.regenerate(0)
+    sc.capture()
+    for it, kv in enumerate((kv0, kv1)):
+        sc.set_kv_len(kv)
+        sc.regenerate(it)
+        sc.run_eager()
+        torch.cuda.synchronize()
+        eager = sc.outputs()
+        eager_lse = [lay.lse.clone() for lay in sc.layers]
+        if it == 0:
+            plain.regenerate(0)
+            plain.run_eager()
+            torch.cuda.synchronize()
+            for lay, other in zip(sc.layers, plain.layers):
+                assert torch.equal(lay.out, other.out), lay.index
+        for lay in sc.layers:
+            lay.out.fill_(-1)
+        # the eager pass wrote this iteration's canvas rows into the caches and rotated q in place: same inputs again
+        sc.regenerate(it)
+        sc.replay()
+        torch.cuda.synchronize()
+        for lay, want, want_lse in zip(sc.layers, eager, eager_lse):
+            assert torch.equal(lay.out, want) and torch.equal(lay.lse, want_lse), (kv, lay.index)
+        for idx in (0, 5, 29):
+            r = schedule_oracle_check(sc, po, idx, [0, 128, 255])
+            assert r["finite"] and r["max_abs"] <= 2e-2 and r["mean_abs"] <= 2e-3 and r["lse_rel"] <= 1e-3, (kv, idx, r)
+    # the two prefixes really gave different rows (the canvas differs too; this guards against a stale device word)
+    assert sc.kv_len == kv1
