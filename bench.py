@@ -842,7 +842,9 @@ def main():
         n_copies = int(min(16, -(-600e6 // kv_alloc_bytes)))
         copies = [kd] + [kd.clone() for _ in range(n_copies - 1)]
         kv_from_hbm = {"copies": n_copies, "cache_bytes": int(kv_alloc_bytes)}
-        for key, flag in (("ms_per_step", 0), ("ms_per_step_with_hint", capi.DG_ATTN_F_KV_FROM_HBM)):
+        # (without a hint the library guesses from what the recent calls streamed, and here it guesses "from HBM")
+        for key, flag in (("ms_per_step_no_touch_ahead", capi.DG_ATTN_F_KV_CACHED), ("ms_per_step", 0),
+                          ("ms_per_step_with_hint", capi.DG_ATTN_F_KV_FROM_HBM)):
             dh = w.desc(n_splits=args.splits, flags=flag | (capi.DG_ATTN_F_STREAMED_MERGE if args.streamed_merge else 0))
             for timed in (False, True):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

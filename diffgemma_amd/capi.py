@@ -18,6 +18,7 @@ DG_ATTN_F_F16_PARTIALS = 0x10
 DG_ATTN_F_STREAMED_MERGE = 0x20
 DG_ATTN_F_KV_FROM_HBM = 0x40
 DG_ATTN_F_SPLIT_OVER_WORKGROUPS = 0x80
+DG_ATTN_F_KV_CACHED = 0x100
 # the reference's DebugStatus vocabulary (debug_status.metal:8-19, dgq_kernels.metal:33-34)
 DG_DBG_ERR_SOFTMAX_NORM_ZERO = 3
 DG_DBG_ERR_NONFINITE = 4

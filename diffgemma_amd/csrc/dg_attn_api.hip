@@ -46,6 +46,37 @@ DeviceInfo g_dev[64];
 thread_local uint32_t* g_tls_dbg = nullptr;
 std::mutex g_dev_mu;
 
+// Which caches this thread's calls streamed lately, to tell whether a call's key/value rows can still be in the
+// memory-side cache (256 MB on MI355X): a cache is taken to be cold when other caches of more than 200 MiB in total
+// were streamed since its last use, or on its first use when it is large.  Decides only which instance of the
+// head_dim 512 kernel runs (the one that touches tiles into the L2 ahead of their loads: same bits, other timing);
+// under graph capture the decision recorded is the one made at capture.
+struct CacheMemo {
+  const void* region = nullptr;
+  uint64_t streamed_at_last_use = 0;
+};
+thread_local CacheMemo g_memo[16];
+thread_local uint64_t g_streamed = 0;
+
+bool cache_is_cold(const void* region, uint64_t bytes) {
+  int idx = -1, oldest = 0;
+  for (int i = 0; i < 16; ++i) {
+    if (g_memo[i].region == region) idx = i;
+    if (g_memo[i].streamed_at_last_use < g_memo[oldest].streamed_at_last_use) oldest = i;
+  }
+  bool cold;
+  if (idx < 0) {
+    cold = bytes >= (32ull << 20);
+    idx = oldest;
+    g_memo[idx].region = region;
+  } else {
+    cold = g_streamed - g_memo[idx].streamed_at_last_use > (200ull << 20);
+  }
+  g_streamed += bytes;
+  g_memo[idx].streamed_at_last_use = g_streamed;
+  return cold;
+}
+
 struct ProfState {
   std::vector<hipEvent_t> ev;
   uint32_t used = 0;
@@ -408,7 +439,11 @@ int fill_params(const dg_attn_desc* d, const Plan& pl, const void* q, const void
   // key/value rows this call streams: more than the 256 MiB memory-side cache holds cannot have
   // stayed there from the previous call, whatever else runs in between (131072 keys: 0.933 -> 0.912 ms)
   const uint64_t kv_streamed = 2ull * d->n_kv_heads * (uint64_t)(pl.tile_end - pl.tile_first) * dg::kBlockN * d->head_dim * 2ull;
-  p.touch_ahead = ((d->flags & DG_ATTN_F_KV_FROM_HBM) || kv_streamed > (256ull << 20)) ? 1u : 0u;
+  // ... and a cache that other large caches were streamed after since its last use has been displaced
+  // (cache_is_cold); DG_ATTN_F_KV_CACHED says the caller knows better
+  const bool cold = cache_is_cold(region, kv_streamed) && hd == 512;   // (every call counts towards what was streamed)
+  p.touch_ahead = ((d->flags & DG_ATTN_F_KV_FROM_HBM) || kv_streamed > (256ull << 20) ||
+                   (cold && !(d->flags & DG_ATTN_F_KV_CACHED))) ? 1u : 0u;
   p.scale_log2 = pl.scale * dg::kLog2e;
   return DG_OK;
 }

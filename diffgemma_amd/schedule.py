@@ -95,9 +95,10 @@ class DenoiseSchedule:
             ad = A.make_desc(canvas, nq, nkv, hd, kv_len, window=window, kv_ring_mask=mask,
                              q_dtype=capi.DG_BF16, kv_dtype=capi.DG_BF16, out_dtype=capi.DG_BF16,
                              layout="head_major", t_cap=slots,
-                             # unit-RMS V rows: far inside the f16 range.  The 30 caches add up to 1.1 GB per
-                             # iteration, four times the memory-side cache: a global layer's rows come from HBM
-                             flags=capi.DG_ATTN_F_F16_PARTIALS | (capi.DG_ATTN_F_KV_FROM_HBM if full else 0))
+                             # unit-RMS V rows: far inside the f16 range.  (The 30 caches add up to 1.1 GB per
+                             # iteration, four times the memory-side cache, so a global layer's rows come from HBM:
+                             # the library sees that by itself from what the calls before it streamed.)
+                             flags=capi.DG_ATTN_F_F16_PARTIALS)
             lay = ScheduleLayer(
                 index=i, full=full, head_dim=hd, n_kv_heads=nkv, slots=slots, ring_mask=mask, window=window,
                 rope_desc=rd, attn_desc=ad,

@@ -84,6 +84,11 @@ typedef enum dg_kernel_sel {
                                               from HBM, 2 % slower when they were cached after all.  Results
                                               are the same bits either way.  A call that streams more than
                                               256 MiB of keys and values does this without being told. */
+#define DG_ATTN_F_KV_CACHED 0x100u         /* hint, the opposite: the rows WILL be in the memory-side cache.  Without either
+                                              hint the library guesses from what the calling thread's recent calls
+                                              streamed: a cache is taken to be displaced when other caches of more than
+                                              200 MiB in total were read since its last use (a loop over a model's
+                                              layers), or on its first use when it is 32 MiB or more. */
 #define DG_ATTN_F_STREAMED_MERGE 0x20u     /* merge the split partial rows with the streaming kernel (weights
                                               first, then only the rows of splits that count) even where the
                                               library would pick the one that fetches every partial row up
