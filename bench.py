@@ -36,6 +36,9 @@ def parse_args():
     ap.add_argument("--global-topk", action="store_true",
                     help="cfg5_schedule: run the global layers as top-k sparse attention (the reference's default for them)")
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--split-over-workgroups", action="store_true",
+                    help="head_dim <= 256, short key range: run the general kernel (keys split over workgroups + merge launch) "
+                         "instead of the one-launch kernel the library picks there")
     ap.add_argument("--streamed-merge", action="store_true",
                     help="merge split partial rows with the streaming kernel even where the up-front one would be picked")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -89,7 +92,7 @@ def cpu_baseline(w, q, kv, flops_per_tok, seconds):
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     "cfg3_global": (152.5e6 + 33.8e6, "profiles/attn_mfma_kernel_cfg3_global_hbm_traffic.md"),
     "cfg4_long": (555.3e6 + 33.8e6, "profiles/attn_mfma_kernel_cfg4_long_hbm_traffic.md"),
-    "cfg2_sliding": (12.9e6 + 12.8e6, "profiles/attn_mfma_kernel_cfg2_sliding_kernel_trace.md"),
+    "cfg2_sliding": (12.9e6 + 2.2e6, "profiles/attn_wsplit_kernel_cfg2_sliding_kernel_trace.md"),
 }
 
 
@@ -674,7 +677,9 @@ def main():
     q, kv = W.generate(w)
     qd, kd = W.device_arrays(w, q, kv)
     t_gen = time.perf_counter() - t_gen
-    desc = w.desc(n_splits=args.splits, flags=capi.DG_ATTN_F_STREAMED_MERGE if args.streamed_merge else 0)
+    base_flags = ((capi.DG_ATTN_F_STREAMED_MERGE if args.streamed_merge else 0) |
+                  (capi.DG_ATTN_F_SPLIT_OVER_WORKGROUPS if args.split_over_workgroups else 0))
+    desc = w.desc(n_splits=args.splits, flags=base_flags)
     pairs, flops = capi.visible_pairs(desc)
     n_splits = capi.resolved_splits(desc)
     out_dt = torch.int16 if w.dtype == "bf16" else torch.float32
@@ -845,7 +850,7 @@ def main():
         # (without a hint the library guesses from what the recent calls streamed, and here it guesses "from HBM")
         for key, flag in (("ms_per_step_no_touch_ahead", capi.DG_ATTN_F_KV_CACHED), ("ms_per_step", 0),
                           ("ms_per_step_with_hint", capi.DG_ATTN_F_KV_FROM_HBM)):
-            dh = w.desc(n_splits=args.splits, flags=flag | (capi.DG_ATTN_F_STREAMED_MERGE if args.streamed_merge else 0))
+            dh = w.desc(n_splits=args.splits, flags=flag | base_flags)
             for timed in (False, True):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
@@ -912,7 +917,8 @@ def main():
                      "frac": kern_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
                      # not read by this run: the counters need the profiler; copied from the committed summary
                      "traffic_source": traffic_source,
-                     "kernel": "attn_mfma_kernel", "kernel_ms": kern_ms,
+                     "kernel": "attn_wsplit_kernel" if n_splits == 1 and w.head_dim <= 256 and not args.splits else "attn_mfma_kernel",
+                     "kernel_ms": kern_ms,
                      "mfma_only_microkernel_tflops": mfma_only_tflops,
                      "frac_of_mfma_only_microkernel": kern_tflops / mfma_only_tflops,
                      "mfma_only_random_operands_tflops": mfma_random_tflops,
