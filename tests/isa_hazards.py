@@ -8,10 +8,12 @@ the emitted assembly in program order and, for every MFMA whose destination is a
 counts wait states until something other than an MFMA accumulating into the very same tuple
 touches one of its registers.
 
-Wait states: one per instruction, n + 1 for `s_nop n`, and PASSES for an MFMA in between (the
-matrix pipe runs a wave's MFMAs in order, one behind the other).  A result may be read PASSES + 3
-wait states after its MFMA.  PASSES is 8 or 16 for the 32x32x16 shapes depending on whom one
-asks: a finding is reported unless the distance holds under both.
+Wait states: one per instruction, n + 1 for `s_nop n`, and 8 for an MFMA in between (a 32x32x16
+MFMA is 8 passes on gfx950, and the matrix pipe runs a wave's MFMAs in order, one behind the
+other).  A result may be read or overwritten 12 wait states after its MFMA: the distance the
+compiler's own hazard recogniser keeps on this target between such an MFMA and a
+`v_accvgpr_read` of its result (it pads with `s_nop` up to exactly that).  MFMAs the compiler
+knows are walked as well: the reader may be assembly (`v_accvgpr_read` of O in the epilogues).
 """
 from __future__ import annotations
 
@@ -19,18 +21,23 @@ import re
 from dataclasses import dataclass
 
 _MFMA = re.compile(r"^\s*v_mfma_\w+\s+(v|a)\[(\d+):(\d+)\]\s*,(.*)$")
-_REG_RANGE = re.compile(r"\bv\[(\d+):(\d+)\]")
-_REG_ONE = re.compile(r"\bv(\d+)\b")
+_REG_RANGE = re.compile(r"\b([va])\[(\d+):(\d+)\]")
+_REG_ONE = re.compile(r"\b([va])(\d+)\b")
 _NOP = re.compile(r"^\s*s_nop\s+(\d+)")
 
 
-def _vgprs(text: str) -> set[int]:
-    regs: set[int] = set()
-    for a, b in _REG_RANGE.findall(text):
-        regs.update(range(int(a), int(b) + 1))
-    for a in _REG_ONE.findall(_REG_RANGE.sub(" ", text)):
-        regs.add(int(a))
+def _vgprs(text: str) -> set:
+    """The vector registers an instruction names: ("v", n) ordinary, ("a", n) accumulation."""
+    regs: set = set()
+    for c, a, b in _REG_RANGE.findall(text):
+        regs.update((c, i) for i in range(int(a), int(b) + 1))
+    for c, a in _REG_ONE.findall(_REG_RANGE.sub(" ", text)):
+        regs.add((c, int(a)))
     return regs
+
+
+def _tuple(cls: str, lo: str, hi: str) -> set:
+    return {(cls, i) for i in range(int(lo), int(hi) + 1)}
 
 
 @dataclass
@@ -70,7 +77,7 @@ def _parse(asm_text: str):
     return funcs
 
 
-_LIMIT = {8: 11, 16: 19}   # wait states before a result may be read or overwritten, by MFMA passes
+_LIMIT = {8: 12}   # MFMA passes -> wait states before its result may be read or overwritten
 _BRANCH = re.compile(r"^\s*s_(c?branch\w*)\s+(\.L\w+)")
 
 
@@ -107,7 +114,7 @@ def _walk(items, labels, pos, dest, have, mfma_line, func, findings, seen):
         m2 = _MFMA.match(text)
         if m2:
             ab, c = m2.group(4).rsplit(",", 1)
-            same = m2.group(1) == "v" and set(range(int(m2.group(2)), int(m2.group(3)) + 1)) == dest
+            same = _tuple(m2.group(1), m2.group(2), m2.group(3)) == dest
             if same and not (_vgprs(ab) & dest) and _vgprs(c) in (dest, set()):
                 return   # accumulates into (or restarts) the same tuple: back to back is fine, and it has its own turn
             if _vgprs(text) & dest:
@@ -121,7 +128,7 @@ def _walk(items, labels, pos, dest, have, mfma_line, func, findings, seen):
         have = {p: have[p] + 1 for p in have}
 
 
-def check(asm_text: str, only_functions: str | None = None) -> list[Finding]:
+def check(asm_text: str, only_functions: str | None = None, all_mfmas: bool = True) -> list[Finding]:
     findings: list[Finding] = []
     for func, items in _parse(asm_text).items():
         if only_functions is not None and not re.search(only_functions, func):
@@ -129,10 +136,10 @@ def check(asm_text: str, only_functions: str | None = None) -> list[Finding]:
         labels = {text: i for i, (kind, text, _) in enumerate(items) if kind == "label"}
         for i, (kind, text, no) in enumerate(items):
             m = _MFMA.match(text) if kind == "ins" else None
-            if not m or m.group(1) != "v":
+            if not m or (m.group(1) != "v" and not all_mfmas):
                 continue
-            dest = set(range(int(m.group(2)), int(m.group(3)) + 1))
-            _walk(items, labels, i + 1, dest, {8: 0, 16: 0}, text, func, findings, set())
+            dest = _tuple(m.group(1), m.group(2), m.group(3))
+            _walk(items, labels, i + 1, dest, {8: 0}, text, func, findings, set())
     return findings
 
 

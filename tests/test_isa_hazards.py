@@ -71,5 +71,9 @@ kernel_b:
 """
     f = H.check(branchy)
     assert len(f) == 1 and "v_add_f32" in f[0].reader
-    # an MFMA with accumulation registers as destination is the compiler's own business
-    assert not H.check("k:\n\tv_mfma_f32_32x32x16_bf16 a[0:15], v[0:3], v[4:7], a[0:15]\n\tv_accvgpr_read_b32 v9, a0\n")
+    # accumulation registers are walked too: the compiler pads its own reads, an assembly read it does not
+    acc = "k:\n\tv_mfma_f32_32x32x16_bf16 a[0:15], v[0:3], v[4:7], a[0:15]\n{}\tv_accvgpr_read_b32 v9, a0\n\ts_endpgm\n"
+    assert len(H.check(acc.format("\ts_nop 3\n"))) == 1
+    assert not H.check(acc.format("\ts_nop 11\n"))
+    # another MFMA in between occupies the matrix pipe for its eight passes
+    assert not H.check(acc.format("\tv_mfma_f32_32x32x16_bf16 a[16:31], v[0:3], v[4:7], a[16:31]\n\ts_nop 3\n"))
