@@ -506,7 +506,8 @@ def other_configs():
     """Short measurements of the other benchmark configurations, run after the headline's timed steps (never
     inside them), the way the reference's bench walks its shapes in one run
     (src/shaders/attn/attention/mod.rs:992-1021): each is checked against the oracle on a few rows, then timed
-    by HIP graph replay (best of a few replays)."""
+    by HIP graph replay (best of a few replays).  Configurations 2, 4 and 5, and configuration 3's shape on the
+    reference's own storage (f16 cache) and on a flat softmax."""
     import torch
     from diffgemma_amd import attention as A, capi, rounding as R, schedule, workloads as W
     from helpers import schedule_oracle_check
@@ -568,6 +569,37 @@ def other_configs():
                          "data": "generated on the device (torch.Generator seed 4)", "check": chk}
     del qd, kd, qb, kvb, ws
     torch.cuda.empty_cache()
+
+    # ---- configuration 3's shape on the two kinds of input the headline does not show (device-generated like
+    # configuration 4): the reference's own storage, bf16 activations over an f16 cache (what dg_attention_dispatch
+    # always runs); and a flat softmax, queries of std 1/sqrt(head_dim) without RMSNorm, so that no weight is
+    # negligible (the headline's unit-RMS rows without a 1/sqrt(d) scale are so peaked that nearly all weights
+    # are stored as exact zeros, which the power-limited matrix cores reward) ----
+    for name in ("cfg3_global_f16kv", "cfg3_global_flat"):
+        w = W.config(name)
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(3)
+        qf = torch.randn(w.canvas, w.n_q_heads, w.head_dim, device="cuda", generator=gen) * w.q_std
+        kvf = torch.randn(2, w.n_kv_heads, w.t_all, w.head_dim, device="cuda", generator=gen)
+        if w.rms_norm:
+            qf = qf * torch.rsqrt(qf.square().mean(-1, keepdim=True) + W.RMS_EPS)
+            kvf = kvf * torch.rsqrt(kvf.square().mean(-1, keepdim=True) + W.RMS_EPS)
+        qb, kvb = qf.to(torch.bfloat16), kvf.to(torch.float16 if w.kv_f16 else torch.bfloat16)
+        del qf, kvf
+        qd, kd = qb.view(torch.int16).reshape(-1), kvb.view(torch.int16).reshape(-1)
+        desc = w.desc()
+        ws = A.alloc_workspace(desc)
+        out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.int16, device="cuda")
+        lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+        A.forward(desc, qd, kd, out, lse, ws)
+        torch.cuda.synchronize()
+        chk = oracle_rows(w, qb.float().cpu().numpy(), kvb.float().cpu().numpy(), out, lse, np.array([5, 200], dtype=np.uint32))
+        ms = _graph_time(lambda: A.forward(desc, qd, kd, out, lse, ws), 40, 5)
+        fl = capi.visible_pairs(desc)[1]
+        recs[name] = {"ms_per_step": ms, "tflops": fl / (ms * 1e-3) / 1e12, "frac": fl / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                      "flops_per_step": fl, "data": "generated on the device (torch.Generator seed 3)", "check": chk}
+        del qd, kd, qb, kvb, ws
+        torch.cuda.empty_cache()
 
     # ---- configuration 5: the 30-layer schedule under a HIP graph, 16 iterations ----
     sc = schedule.DenoiseSchedule().build()
