@@ -129,6 +129,10 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
   const bool active = d0 < hd;
   float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (active) load_row<PER>(src + d0, x);
+  // (the norm weights too, now: asked for where they are used, behind the row sum, they were a second trip to
+  // memory on the wave's critical path)
+  float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (active && (is_q || is_k)) load_row<PER>((is_q ? p.qw : p.kw) + d0, w);
   // The angles depend on the position only: the workgroup's four heads share one table of cos and sin,
   // one pair per thread, worked out while the rows are on their way (rotation, cpu.rs:31-65: pairs
   // (d, hd/2 + d) for d < rot/2; split-half: rot = hd, theta 1e4; proportional: rot = hd/4, theta 1e6,
@@ -162,8 +166,6 @@ __global__ void __launch_bounds__(256) qk_rope_kv_kernel(const RopeParams p) {
 
   float* st = stage[wave];
   if (active) {
-    float w[8];
-    load_row<PER>((is_q ? p.qw : p.kw) + d0, w);
 #pragma unroll
     for (int i = 0; i < PER; ++i) st[d0 + i] = x[i] * (inv * w[i]);   // x * (inv * w), the CPU twin's order (cpu.rs:71-74)
   }
