@@ -317,6 +317,25 @@ class AttnRig:
                                              C.byref(lo), C.byref(sp), C.byref(dims), self.buf_dbg.data_ptr(),
                                              st.data_ptr(), st.numel(), stream_handle()))
 
+    def run_dispatch_dev(self, *, causal: int = 0, window: int = 0, kv_len_max: Optional[int] = None) -> None:
+        """run_dispatch with StepParams bound as the reference binds it (enc.rs:2177-2220, buf4): a device buffer
+        whose kv_len the kernels read when they run; the host only says how far the prefix can grow."""
+        f = self.fixture
+        lib = capi.load()
+        lo = layer_offsets(f, self.kv_ring_mask)
+        kv_len_max = f.kv_len if kv_len_max is None else kv_len_max
+        self.step_dev = device_step_params(f.kv_len)
+        dims = capi.AttnDims(canvas=f.canvas, n_q_heads=f.n_q_heads, causal=causal, window=window)
+        n = C.c_size_t(0)
+        capi.check(lib.dg_attention_state_bytes(C.byref(lo), C.byref(dims), kv_len_max, C.byref(n)))
+        key = ("state", n.value)
+        if key not in self._ws:
+            self._ws[key] = _torch().empty(max(n.value, 256), dtype=_torch().uint8, device="cuda")
+        st = self._ws[key]
+        capi.check(lib.dg_attention_dispatch_dev(self.buf_q.data_ptr(), self.buf_kv.data_ptr(), self.buf_out.data_ptr(),
+                                                 C.byref(lo), self.step_dev.data_ptr(), kv_len_max, C.byref(dims),
+                                                 self.buf_dbg.data_ptr(), st.data_ptr(), st.numel(), stream_handle()))
+
     def time_rounds(self, iters: int, encode, rounds: int = 6):
         """6 rounds of `iters` back-to-back launches, round 0 discarded; returns
         (min, median) mean-ms-per-launch over the kept rounds (harness.rs:149-170)."""

@@ -169,6 +169,19 @@ class RopeRig:
             A.stream_handle()))
         A._torch().cuda.synchronize()
 
+    def run_dispatch_dev(self) -> None:
+        """run_dispatch with StepParams as a device buffer (qk_rope_kv.metal:30-38 binds it so): kv_len and
+        kv_write_end are read when the kernel runs."""
+        f = self.f
+        L = layer_offsets(f)
+        self.step_dev = A.device_step_params(f.kv_len, f.kv_write_end)
+        dims = capi.AttnDims(f.canvas, f.n_q_heads, 0, 0)
+        capi.check(capi.load().dg_qk_rope_kv_dispatch_dev(
+            self.buf_q.data_ptr(), self.buf_k.data_ptr(), self.buf_v.data_ptr(), self.buf_kv.data_ptr(),
+            self.buf_blob.data_ptr(), C.byref(L), self.step_dev.data_ptr(), C.byref(dims), self.buf_dbg.data_ptr(),
+            A.stream_handle()))
+        A._torch().cuda.synchronize()
+
     def read(self):
         """(q, k, kvcache) as f32 host arrays."""
         q = rounding.bf16_bits_to_f32(self.buf_q.cpu().numpy().view(np.uint16))

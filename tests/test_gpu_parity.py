@@ -54,6 +54,26 @@ def test_reference_fixture_mfma_dispatch(gpu_ready, po, name, causal):
 
 
 @pytest.mark.parametrize("name", list(FIXTURES))
+@pytest.mark.parametrize("causal", [0, 1])
+def test_reference_fixture_dispatch_with_device_step_params(gpu_ready, po, name, causal):
+    """dg_attention_dispatch_dev: StepParams bound as a device buffer (enc.rs:2177-2220), kv_len read when the
+    kernels run.  Planned for exactly this prefix it gives the host-P entry's bits; planned for a longer one
+    (the split plan then differs) it still meets the oracle."""
+    fn, tol = FIXTURES[name]
+    f = fn()
+    want, _, _ = reference_cpu(po, f, causal_rows=f.canvas if causal else 0)
+    host, dev = A.AttnRig.from_fixture(f), A.AttnRig.from_fixture(f)
+    host.run_dispatch(causal=causal)
+    dev.run_dispatch_dev(causal=causal)
+    assert np.array_equal(host.read_out_f32().view(np.uint32), dev.read_out_f32().view(np.uint32))
+    slack = 4096      # slots the cache buffer holds behind the fixture's rows: the plan may reach that far
+    far = A.AttnRig.from_fixture(f, kv_slack_slots=slack)
+    far.run_dispatch_dev(causal=causal, kv_len_max=f.kv_len + slack)
+    assert_oracle(far.read_out_f32(), want, tol, 0.9999)
+    assert dev.read_debug_status().code == 0 and far.read_debug_status().code == 0
+
+
+@pytest.mark.parametrize("name", list(FIXTURES))
 def test_reference_fixture_unrounded_and_lse(gpu_ready, po, name):
     import torch
     f = FIXTURES[name][0]()

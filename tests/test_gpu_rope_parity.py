@@ -109,6 +109,27 @@ def test_write_suppression_and_untouched_rows(gpu_ready, po):
     assert max_abs_diff(gq, q) <= 2e-2 and max_abs_diff(gkv, kvc) <= 1e-2   # suppressed rows still rotate q
 
 
+@pytest.mark.parametrize("name", ["tiny", "full_hd512_v_alias"])
+def test_dispatch_with_device_step_params_equals_the_host_one(gpu_ready, name):
+    """dg_qk_rope_kv_dispatch_dev reads kv_len and kv_write_end from a device StepParams when the kernel runs
+    (the reference binds StepParams as a device buffer, qk_rope_kv.metal:30-38): same bits as the host-P entry,
+    including a kv_write_end that suppresses part of the canvas."""
+    f = CASES[name][0]()
+    a, b = QR.RopeRig(f), QR.RopeRig(f)
+    a.run_dispatch()
+    b.run_dispatch_dev()
+    for x, y in zip(a.read(), b.read()):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+    f2 = QR.random_fixture(8, 16, 8, 256, 1020, is_full=False, v_proj=1, seed=9, kv_ring_mask=1023, kv_write_end=1024,
+                           kv_region=4096)
+    a, b = QR.RopeRig(f2), QR.RopeRig(f2)
+    a.run_dispatch()
+    b.run_dispatch_dev()
+    for x, y in zip(a.read(), b.read()):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+    assert b.buf_dbg.cpu().numpy()[0] == 0
+
+
 def test_general_entry_bf16_head_major_cache(gpu_ready, po):
     """dg_qk_rope_kv with the cache the benchmark's attention reads: bf16, two planes [Hkv][t_cap][d]."""
     import torch
