@@ -137,6 +137,15 @@ def load():
         raise RuntimeError(
             f"{path} is missing: build it with `python -m diffgemma_amd.build` (needs hipcc); "
             "there is no CPU fallback for the attention path")
+    # One HIP runtime per process.  PyTorch brings its own libamdhip64.so.7 and the library was linked against the
+    # system's, same soname: the dynamic loader gives every later user whichever copy came first.  The tensors this
+    # package hands to the library are PyTorch's, so PyTorch's runtime has to be that copy: loaded the other way
+    # round, the first launch fails with DG_ERR_DEVICE ("no gfx950 device current").  (A C or Rust host links one
+    # runtime and has no such choice to make.)
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(str(path))
     P, VP = C.POINTER, C.c_void_p
     lib.dg_attn_desc_reference_layout.argtypes = [P(AttnDesc)]
