@@ -72,6 +72,37 @@ def test_layer_shapes(gpu_ready, po, shape):
     assert ds[0] == 0, f"debug status {ds}"
 
 
+def _random_case(seed):
+    rng = np.random.default_rng(5000 + seed)
+    hd = int(rng.choice([32, 64, 128, 256, 512]))
+    nkv = int(rng.choice([1, 2, 4, 8]))
+    nq = nkv * int(rng.choice([1, 2, 4, 8]))
+    canvas = int(rng.choice([1, 3, 16, 37, 64, 256]))
+    ring = int(rng.choice([0, 0, 255, 1023, 2047]))
+    kv_len = int(rng.choice([0, 1, 100, 1000, 5000, 40000])) if ring == 0 else int(rng.choice([0, 100, 1000, 70000]))
+    canvas = min(canvas, ring + 1) if ring else canvas
+    is_full, v_proj = bool(rng.integers(0, 2)), int(rng.integers(0, 2))
+    kv_write_end = 0xFFFFFFFF if rng.random() < 0.6 else kv_len + int(rng.integers(0, canvas + 1))
+    return QR.random_fixture(canvas, nq, nkv, hd, kv_len, is_full=is_full, v_proj=v_proj, seed=seed, kv_ring_mask=ring,
+                             kv_write_end=kv_write_end, kv_region=int(rng.choice([0, 4096])))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes(gpu_ready, po, seed):
+    """Seeded sweep over head_dim, head counts, ragged canvases, rings, prefixes, both rotations, V aliasing and
+    write suppression, through both reference-shaped entries (host and device StepParams)."""
+    f = _random_case(seed)
+    q, k, kvc = reference_cpu(po, f)
+    for dev in (False, True):
+        rig = QR.RopeRig(f)
+        (rig.run_dispatch_dev if dev else rig.run_dispatch)()
+        gq, gk, gkv = rig.read()
+        assert np.isfinite(gq).all() and np.isfinite(gkv).all()
+        assert np.all(np.abs(gq - q) <= storage_tolerance(q, 7)) and np.all(np.abs(gk - k) <= storage_tolerance(k, 7))
+        assert np.all(np.abs(gkv - kvc) <= storage_tolerance(kvc, 10))
+        assert rig.buf_dbg.cpu().numpy()[0] == 0
+
+
 def test_debug_status_names_the_producer(gpu_ready):
     """A NaN in one head's input makes that head's 1/rms non-finite; the record the kernel leaves is the
     reference's: DbgErrNonFinite = 4 in DbgKernelQkRopeKv = 25, value = the canvas row
