@@ -62,15 +62,15 @@ __device__ __forceinline__ void mfma_scores_acc(f32x16& s, u32x4 a, u32x4 b) {
   if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
   else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
 }
-// Last score MFMA of a tile, followed by 24 wait states: more than the 20 a 16-pass MFMA result
-// needs before a VALU may read it.  They are part of the same asm statement so that no
-// compiler-made register copy of the scores can land between the MFMA and the wait.
+// Last score MFMA of a tile, followed by 12 wait states: what the compiler's own hazard recogniser keeps between
+// an MFMA of this shape (8 passes) and a VALU read of its result on this target.  They are part of the same asm
+// statement so that no compiler-made register copy of the scores can land between the MFMA and the wait.
 template <bool F16>
 __device__ __forceinline__ void mfma_scores_last(f32x16& s, u32x4 a, u32x4 b) {
   if constexpr (F16)
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 11" : "+v"(s) : "v"(a), "v"(b));
   else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 7" : "+v"(s) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 11" : "+v"(s) : "v"(a), "v"(b));
 }
 
 // x *= c for values that live in accumulation registers, without the register allocator moving
