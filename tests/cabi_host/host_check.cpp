@@ -1,0 +1,252 @@
+// A host program with no Python and no PyTorch in it: it links the library through include/dg_attn.h the way the
+// reference's Rust side would through its FFI (one HIP runtime, the system's), runs the attention entry points on
+// seeded inputs and compares with the CPU oracle (test infrastructure, linked here as the checker only).
+// Exit status 0 = every case within the tolerance the parity tests use; the lines it prints name each case.
+//
+//   case A  global-layer shape, bf16 head-major cache, mixed mask, splits + merge   (dg_attn_forward)
+//   case B  sliding-layer shape, window 1024 on a ring cache, one launch            (dg_attn_forward, no workspace)
+//   case C  the reference's own argument block: bf16 q, f16 slot-major cache        (dg_attention_dispatch, causal = 1)
+//   case D  case A through the entry that allocates nothing                         (dg_attn_forward_static)
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../include/dg_attn.h"
+#include "../../oracle/dg_attn_oracle.h"
+
+#define HIP_OK(x)                                                                   \
+  do {                                                                              \
+    hipError_t e_ = (x);                                                            \
+    if (e_ != hipSuccess) {                                                         \
+      std::printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+      return 2;                                                                     \
+    }                                                                               \
+  } while (0)
+#define DG_OK_(x)                                                                   \
+  do {                                                                              \
+    int s_ = (x);                                                                   \
+    if (s_ != DG_OK) {                                                              \
+      std::printf("dg_attn status %d (%s) at %s:%d\n", s_, dg_attn_strerror(s_), __FILE__, __LINE__); \
+      return 3;                                                                     \
+    }                                                                               \
+  } while (0)
+
+namespace {
+
+struct Rng {   // xorshift64*, then Box-Muller
+  uint64_t s;
+  explicit Rng(uint64_t seed) : s(seed * 0x9E3779B97F4A7C15ull + 1) {}
+  uint64_t next() {
+    s ^= s >> 12;
+    s ^= s << 25;
+    s ^= s >> 27;
+    return s * 0x2545F4914F6CDD1Dull;
+  }
+  double uniform() { return ((next() >> 11) + 0.5) * (1.0 / 9007199254740992.0); }
+  float normal() { return (float)(std::sqrt(-2.0 * std::log(uniform())) * std::cos(6.283185307179586 * uniform())); }
+};
+
+uint16_t bf16_rne(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+float bf16_val(uint16_t h) {
+  uint32_t u = (uint32_t)h << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+uint16_t f16_rne(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+float f16_val(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+
+// rows of `hd` elements with unit RMS (what a cache holds after the producer's RMSNorm)
+void unit_rms_rows(Rng& rng, std::vector<float>& x, size_t rows, size_t hd) {
+  x.resize(rows * hd);
+  for (size_t r = 0; r < rows; ++r) {
+    double ss = 0;
+    for (size_t i = 0; i < hd; ++i) {
+      x[r * hd + i] = rng.normal();
+      ss += (double)x[r * hd + i] * x[r * hd + i];
+    }
+    const float inv = (float)(1.0 / std::sqrt(ss / hd + 1e-6));
+    for (size_t i = 0; i < hd; ++i) x[r * hd + i] *= inv;
+  }
+}
+
+struct Shape {
+  const char* name;
+  uint32_t canvas, hq, hkv, hd, kv_len, causal_rows, window, ring_mask;
+  bool reference_args;   // case C: dg_attention_dispatch with an f16 slot-major cache
+  bool static_entry;     // case D
+};
+
+int run(const Shape& sh, uint64_t seed, hipStream_t stream) {
+  Rng rng(seed);
+  const uint32_t t_all = sh.kv_len + sh.canvas;
+  const uint32_t slots = sh.ring_mask ? sh.ring_mask + 1u : t_all;
+  std::vector<float> q, kv;
+  unit_rms_rows(rng, q, (size_t)sh.canvas * sh.hq, sh.hd);
+  unit_rms_rows(rng, kv, (size_t)2 * sh.hkv * slots, sh.hd);   // two planes or slot-major: the same number of rows
+
+  // storage rounding on the host; the oracle sees the rounded values
+  std::vector<uint16_t> qb(q.size()), kvb(kv.size());
+  for (size_t i = 0; i < q.size(); ++i) {
+    qb[i] = bf16_rne(q[i]);
+    q[i] = bf16_val(qb[i]);
+  }
+  for (size_t i = 0; i < kv.size(); ++i) {
+    kvb[i] = sh.reference_args ? f16_rne(kv[i]) : bf16_rne(kv[i]);
+    kv[i] = sh.reference_args ? f16_val(kvb[i]) : bf16_val(kvb[i]);
+  }
+
+  dgo_desc od;
+  std::memset(&od, 0, sizeof od);
+  od.canvas = sh.canvas;
+  od.n_q_heads = sh.hq;
+  od.n_kv_heads = sh.hkv;
+  od.head_dim = sh.hd;
+  od.kv_len = sh.kv_len;
+  od.causal_rows = sh.causal_rows;
+  od.window = sh.window;
+  od.kv_ring_mask = sh.ring_mask;
+  od.t_lo_override = -1;
+  od.scale = 1.0f;
+  if (sh.reference_args) dgo_desc_reference_layout(&od);
+  else dgo_desc_head_major_layout(&od, slots);
+  const size_t n_out = (size_t)sh.canvas * sh.hq * sh.hd, n_rows = (size_t)sh.canvas * sh.hq;
+  std::vector<float> ref(n_out), ref_lse(n_rows);
+  dgo_attention_f32(&od, q.data(), kv.data(), ref.data(), ref_lse.data(), nullptr, 0, 0);
+  if (sh.reference_args)   // the reference's wrapper stores its CPU result as bf16 by truncation (attention/mod.rs:218-240),
+    for (float& x : ref) {  // as its kernels and this library's dispatch entry store theirs
+      uint32_t u;
+      std::memcpy(&u, &x, 4);
+      u &= 0xffff0000u;
+      std::memcpy(&x, &u, 4);
+    }
+
+  void *dq = nullptr, *dkv = nullptr, *dout = nullptr, *dlse = nullptr, *dws = nullptr, *ddbg = nullptr;
+  HIP_OK(hipMalloc(&dq, qb.size() * 2));
+  HIP_OK(hipMalloc(&dkv, kvb.size() * 2 + 64 * 1024));   // (slack behind the cache, as the reference's buffers have)
+  HIP_OK(hipMalloc(&dout, n_out * 2));
+  HIP_OK(hipMalloc(&dlse, n_rows * 4));
+  HIP_OK(hipMalloc(&ddbg, 16));
+  HIP_OK(hipMemset(dkv, 0, kvb.size() * 2 + 64 * 1024));
+  HIP_OK(hipMemset(ddbg, 0, 16));
+  HIP_OK(hipMemcpy(dq, qb.data(), qb.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(dkv, kvb.data(), kvb.size() * 2, hipMemcpyHostToDevice));
+
+  bool have_lse = true;
+  if (sh.reference_args) {
+    dg_layer_offsets L;
+    std::memset(&L, 0, sizeof L);
+    L.head_dim = sh.hd;
+    L.n_kv_heads = sh.hkv;
+    L.is_full = sh.hd == 512;
+    L.kv_ring_mask = sh.ring_mask;
+    dg_step_params P;
+    std::memset(&P, 0, sizeof P);
+    P.kv_len = sh.kv_len;
+    P.kv_write_end = 0xffffffffu;
+    dg_attn_dims dims = {sh.canvas, sh.hq, sh.causal_rows == sh.canvas ? 1u : 0u, sh.window};
+    size_t state_bytes = 0;
+    DG_OK_(dg_attention_state_bytes(&L, &dims, sh.kv_len, &state_bytes));
+    HIP_OK(hipMalloc(&dws, state_bytes ? state_bytes : 256));
+    DG_OK_(dg_attention_dispatch(dq, dkv, dout, &L, &P, &dims, (dg_debug_status*)ddbg, dws, state_bytes, stream));
+    have_lse = false;   // the reference's entry has no LSE output
+  } else {
+    dg_attn_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.canvas = sh.canvas;
+    d.n_q_heads = sh.hq;
+    d.n_kv_heads = sh.hkv;
+    d.head_dim = sh.hd;
+    d.kv_len = sh.kv_len;
+    d.causal_rows = sh.causal_rows;
+    d.window = sh.window;
+    d.kv_ring_mask = sh.ring_mask;
+    d.q_dtype = d.kv_dtype = d.out_dtype = DG_BF16;
+    d.flags = DG_ATTN_F_F16_PARTIALS;   // unit-RMS V rows: far inside the f16 range
+    dg_attn_desc_head_major_layout(&d, slots);
+    size_t ws_bytes = 0;
+    DG_OK_(dg_attn_workspace_bytes(&d, &ws_bytes));
+    uint32_t splits = 0;
+    DG_OK_(dg_attn_resolved_splits(&d, &splits));
+    std::printf("  %s: %u split(s), workspace %zu bytes\n", sh.name, splits, ws_bytes);
+    if (sh.static_entry) {
+      DG_OK_(dg_attn_forward_static(&d, dq, dkv, dout, (float*)dlse, stream));
+    } else {
+      HIP_OK(hipMalloc(&dws, ws_bytes ? ws_bytes : 256));
+      DG_OK_(dg_attn_forward(&d, dq, dkv, dout, (float*)dlse, dws, ws_bytes, stream));
+    }
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+
+  std::vector<uint16_t> ob(n_out);
+  std::vector<float> lse(n_rows);
+  uint32_t dbg[4];
+  HIP_OK(hipMemcpy(ob.data(), dout, n_out * 2, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(lse.data(), dlse, n_rows * 4, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(dbg, ddbg, 16, hipMemcpyDeviceToHost));
+  double max_abs = 0, sum_abs = 0, lse_rel = 0;
+  bool finite = true;
+  for (size_t i = 0; i < n_out; ++i) {
+    const float g = bf16_val(ob[i]);
+    finite = finite && std::isfinite(g);
+    const double e = std::fabs((double)g - ref[i]);
+    max_abs = e > max_abs ? e : max_abs;
+    sum_abs += e;
+  }
+  if (have_lse)
+    for (size_t r = 0; r < n_rows; ++r) {
+      const double e = std::fabs((double)lse[r] - ref_lse[r]) / std::fabs((double)ref_lse[r]);
+      lse_rel = e > lse_rel ? e : lse_rel;
+    }
+  const double mean_abs = sum_abs / n_out;
+  const bool ok = finite && max_abs <= 2e-2 && mean_abs <= 2e-3 && lse_rel <= 1e-3 && dbg[0] == 0;
+  std::printf("%s %s: max_abs %.3e mean_abs %.3e lse_rel %.3e debug code %u\n", ok ? "PASS" : "FAIL", sh.name, max_abs,
+              mean_abs, lse_rel, dbg[0]);
+  std::fflush(stdout);
+  (void)hipFree(dq);
+  (void)hipFree(dkv);
+  (void)hipFree(dout);
+  (void)hipFree(dlse);
+  (void)hipFree(ddbg);
+  if (dws) (void)hipFree(dws);
+  return ok ? 0 : 1;
+}
+
+}  // namespace
+
+int main() {
+  int n_dev = 0;
+  if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
+    std::printf("no HIP device\n");
+    return 4;
+  }
+  HIP_OK(hipSetDevice(0));
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  std::printf("dg_attn ABI version %u\n", dg_attn_abi_version());
+  const Shape shapes[] = {
+      {"A global, mixed mask, splits + merge", 64, 16, 2, 512, 3000, 32, 0, 0, false, false},
+      {"B sliding, ring cache, one launch", 64, 16, 8, 256, 5000, 0, 1024, 2047, false, false},
+      {"C reference argument block, f16 cache, causal", 64, 16, 2, 512, 700, 64, 0, 0, true, false},
+      {"D case A without allocating", 64, 16, 2, 512, 3000, 32, 0, 0, false, true},
+  };
+  int bad = 0;
+  uint64_t seed = 11;
+  for (const Shape& sh : shapes) {
+    const int rc = run(sh, seed++, stream);
+    if (rc > 1) return rc;
+    bad += rc;
+  }
+  HIP_OK(hipStreamDestroy(stream));
+  std::printf(bad ? "%d case(s) failed\n" : "all cases passed\n", bad);
+  return bad ? 1 : 0;
+}
