@@ -31,6 +31,22 @@ def test_library_exports_every_declared_symbol():
     assert lib.dg_attn_abi_version() == 1
 
 
+def test_headers_are_plain_c(tmp_path):
+    """include/*.h is what a foreign-function generator (bindgen, cgo) reads: it has to be C, not C++."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "hdr.c"
+    src.write_text('#include "dg_attn.h"\n#include "dg_attn_bench.h"\n'
+                   "int main(void) { dg_attn_desc d; dg_rope_desc r; dg_layer_offsets l; (void)d; (void)r; (void)l; "
+                   "return sizeof(dg_step_params) == 48 && sizeof(dg_attn_dims) == 16 ? 0 : 1; }\n")
+    res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                          str(src), "-o", str(tmp_path / "hdr")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout
+    assert subprocess.run([str(tmp_path / "hdr")]).returncode == 0
+
+
 def test_flag_constants_match_the_header():
     """The ctypes binding spells the desc.flags bits out again: they must be the header's."""
     text = open(os.path.join(ROOT, "include", "dg_attn.h")).read()
