@@ -672,3 +672,51 @@ def test_hip_graph_replay(gpu_ready):
         assert torch.equal(out_g, out_e), i
         A.forward(d, qd, kd, out_e, None, ws)     # eager work between replays
         torch.cuda.synchronize()
+
+
+def test_two_host_threads_on_two_streams(gpu_ready):
+    """The library keeps no state that two callers share (plans are made per call; the cache memo and the
+    profiling state are per thread): two host threads, each on a stream of its own with buffers of its own,
+    calling in a loop at the same time get the bits a single caller gets.  (The entry that allocates nothing
+    is the documented exception: its scratch is one per GPU.)"""
+    import threading
+    import torch
+    shapes = [W.Workload("thr_a", 64, 16, 2, 512, 3000, causal_rows=32, seed=41),      # splits + merge
+              W.Workload("thr_b", 64, 16, 8, 256, 2000, window=1024, seed=42)]          # one launch
+    want = []
+    for w in shapes:
+        q, kv = W.generate(w)
+        qd, kd = W.device_arrays(w, q, kv)
+        d = w.desc()
+        out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.int16, device="cuda")
+        lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+        A.forward(d, qd, kd, out, lse, A.alloc_workspace(d))
+        torch.cuda.synchronize()
+        want.append((d, qd, kd, out.clone(), lse.clone()))
+    errors = []
+
+    def worker(order):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                bufs = [(torch.zeros_like(o), torch.zeros_like(l), A.alloc_workspace(d)) for d, _, _, o, l in want]
+                for it in range(40):
+                    i = order[it % 2]
+                    d, qd, kd, o_ref, l_ref = want[i]
+                    o, l, ws = bufs[i]
+                    o.zero_()
+                    A.forward(d, qd, kd, o, l, ws)
+                    if it % 8 == 7 or it >= 38:
+                        stream.synchronize()
+                        if not (torch.equal(o, o_ref) and torch.equal(l, l_ref)):
+                            errors.append((order, it, i))
+                stream.synchronize()
+        except Exception as e:   # a failure in a thread must fail the test
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(o,)) for o in ((0, 1), (1, 0))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
