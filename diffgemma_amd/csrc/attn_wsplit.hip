@@ -168,13 +168,18 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
   // the first one, when the range starts inside it, and the last one, when the keys end inside it): block
   // blk covers rows blk * 64 / CPR ..., lane l the 16-byte chunk l of the block, swizzled.  Worked out once;
   // the tile's base address is scalar.
+  // The loads go out in groups that share one setting of M0 (lds_dma_16_group): a quarter of a K tile (its
+  // loads are spread over the softmax in quarters), two blocks of a V tile (two go between each pair of score
+  // MFMAs); the offsets carry the group's bias.
+  constexpr int GK = NBLK >= 4 ? NBLK / 4 : 1, GV = 2;
+  static_assert(NBLK % GK == 0 && NBLK % GV == 0 && GK <= 4, "groups tile the blocks");
   uint32_t koff[NBLK], voff[NBLK];
 #pragma unroll
   for (int blk = 0; blk < NBLK; ++blk) {
     const uint32_t pch = blk * 64 + lane;
     const uint32_t rr_ = pch / L::CPR, pc = pch % L::CPR;
-    koff[blk] = rr_ * (uint32_t)kstride_b + ((pc ^ L::swz_k(rr_)) << 4);
-    voff[blk] = rr_ * (uint32_t)vstride_b + ((pc ^ L::swz_v(rr_)) << 4);
+    koff[blk] = rr_ * (uint32_t)kstride_b + ((pc ^ L::swz_k(rr_)) << 4) + kDmaBias - (uint32_t)(blk % GK) * 1024u;
+    voff[blk] = rr_ * (uint32_t)vstride_b + ((pc ^ L::swz_v(rr_)) << 4) + kDmaBias - (uint32_t)(blk % GV) * 1024u;
   }
   // a tile with rows that must not be read (before the first visible key: dead ring slots; past the last key)
   auto tile_is_edge = [&](uint32_t tile) { return tile * kBlockN < lo_min || tile * kBlockN + kBlockN > p.t_all; };
@@ -187,25 +192,28 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
       const uint32_t pch = blk * 64 + lane;
       const uint32_t rr_ = pch / L::CPR, pc = pch % L::CPR;
       const uint32_t c = pc ^ (IS_V ? L::swz_v(rr_) : L::swz_k(rr_));
-      tab[blk] = min(max(rr_, tl.rmin), tl.rmax) * tl.stride_b + c * 16u;
+      tab[blk] = min(max(rr_, tl.rmin), tl.rmax) * tl.stride_b + c * 16u + kDmaBias - (uint32_t)(blk % (IS_V ? GV : GK)) * 1024u;
     }
   };
-  auto issue_block = [&](auto blk_c, const TileLoad& tl, const uint32_t (&tab)[NBLK]) {
-    constexpr int blk = decltype(blk_c)::value;
-    lds_dma_16<blk * 1024>(tl.base, tab[blk], tl.lds);
+  // group g of a tile's loads: blocks g G .. g G + G - 1
+  auto issue_group = [&](auto is_v_c, auto g_c, const TileLoad& tl, const uint32_t (&tab)[NBLK]) {
+    constexpr int G = decltype(is_v_c)::value ? GV : GK;
+    constexpr int g = decltype(g_c)::value;
+    lds_dma_16_group<G, g * G * 1024>(tl.base - kDmaBias, &tab[g * G], tl.lds);
   };
   using IsK = std::false_type;
   using IsV = std::true_type;
+  constexpr int NGK = NBLK / GK, NGV = NBLK / GV;
 
   // ---- the first K and V tiles are on their way before anything waits for the query rows ----
   if (ntile > 0) {
     uint32_t tab[NBLK];
     const TileLoad ktl0 = k_load(tb);
     edge_table(IsK{}, ktl0, tab);
-    static_for<0, NBLK>([&](auto b_c) { issue_block(b_c, ktl0, tab); });
+    static_for<0, NGK>([&](auto g_c) { issue_group(IsK{}, g_c, ktl0, tab); });
     const TileLoad vtl0 = v_load(tb);
     edge_table(IsV{}, vtl0, tab);
-    static_for<0, NBLK>([&](auto b_c) { issue_block(b_c, vtl0, tab); });
+    static_for<0, NGV>([&](auto g_c) { issue_group(IsV{}, g_c, vtl0, tab); });
   }
 
   // ---- Q fragments: B operand of S^T = K.Q^T, lane = row, 8 consecutive d per step.  The 32 rows come in
@@ -351,7 +359,7 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
     }
     auto k_loads = [&](auto q_c) {   // a quarter of the next K tile's loads
       constexpr int q = decltype(q_c)::value;
-      if (more) static_for<q * NBLK / 4, (q + 1) * NBLK / 4>([&](auto b_c) { issue_block(b_c, ktl, ktab); });
+      if (more) static_for<q * NGK / 4, (q + 1) * NGK / 4>([&](auto g_c) { issue_group(IsK{}, g_c, ktl, ktab); });
     };
 
     // ---- online softmax with a lazily raised reference max ----
@@ -441,8 +449,7 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
       }
       scores([&](auto st_c) {
         constexpr int st = decltype(st_c)::value;
-        if constexpr (2 * st < NBLK) issue_block(std::integral_constant<int, 2 * st>{}, vtl, vtab);
-        if constexpr (2 * st + 1 < NBLK) issue_block(std::integral_constant<int, 2 * st + 1>{}, vtl, vtab);
+        if constexpr (st < NGV) issue_group(IsV{}, st_c, vtl, vtab);
       });
     }
   }

@@ -261,6 +261,36 @@ __device__ __forceinline__ void lds_dma_16(const char* base_uniform, uint32_t vo
   }
 }
 
+// G consecutive KiB blocks of a tile with one setting of M0: block g goes to LDS byte (lds_dst + LDS_IMM) + 1024 g
+// + 16 * l.  The instruction's immediate offset moves the LDS address AND the memory address, so the caller's
+// per-lane offsets are biased: voff[g] = (byte offset from the tile's base) + kDmaBias - 1024 g, and the base passed
+// here is the tile's base minus kDmaBias (the bias keeps every voff non-negative whatever row a clamp picked).
+// Saves an M0 write and the wait state behind it for every block but the first.
+constexpr uint32_t kDmaBias = 4096;
+template <int G, int LDS_IMM>
+__device__ __forceinline__ void lds_dma_16_group(const char* base_minus_bias_uniform, const uint32_t* voff,
+                                                 uint32_t lds_dst_uniform) {
+  static_assert(G == 1 || G == 2 || G == 4, "immediate offsets reach 3 KiB");
+  const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_dst_uniform);
+  const uint64_t base = uniform_address(base_minus_bias_uniform);
+  if constexpr (G == 1) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff[0]), "s"(base),
+                 "n"(LDS_IMM)
+                 : "memory", "scc");
+  } else if constexpr (G == 2) {
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3\n\t"
+                 "global_load_lds_dwordx4 %2, %3 offset:1024" ::"s"(dst),
+                 "v"(voff[0]), "v"(voff[1]), "s"(base), "n"(LDS_IMM)
+                 : "memory", "scc");
+  } else {
+    asm volatile("s_add_u32 m0, %0, %6\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %5\n\t"
+                 "global_load_lds_dwordx4 %2, %5 offset:1024\n\tglobal_load_lds_dwordx4 %3, %5 offset:2048\n\t"
+                 "global_load_lds_dwordx4 %4, %5 offset:3072" ::"s"(dst),
+                 "v"(voff[0]), "v"(voff[1]), "v"(voff[2]), "v"(voff[3]), "s"(base), "n"(LDS_IMM)
+                 : "memory", "scc");
+  }
+}
+
 // lane l: 4 bytes from base + voff -> a dump area in LDS (64 words) that nobody reads.  What the load
 // is for is its side effect: the 128-byte line it touches is in the L2 afterwards.  A load without a
 // register destination, so nothing has to stay reserved until it lands.
