@@ -13,9 +13,10 @@
 // waits only for its own loads (vmcnt): the tile loop has no workgroup barrier.  The score accumulator
 // holds, per lane, 16 keys of the lane's row in exactly the order the B operand of O^T += V^T.P^T wants
 // them, so P never leaves the registers.  K and V have one buffer each per wave (two would not fit the
-// LDS): per tile a wave runs softmax(j) with the loads of K(j+1) spread through it (the K buffer is free
-// once the scores of tile j exist), then P.V(j), then the scores of tile j+1 with the loads of V(j+1)
-// between its first MFMAs (the V buffer is free after P.V).  Each load has about half a tile's time to land.
+// LDS): per tile a wave runs softmax(j), with the loads of K(j+1) issued as soon as the tile's maximum has
+// read the scores (the K buffer is free once the scores of tile j exist), then P.V(j), then the scores of tile
+// j+1 with the loads of V(j+1) between its middle MFMAs (the V buffer is free after P.V).  A tile's loads go out
+// in groups under one setting of M0 (the instruction's immediate offset moves the LDS address as well).
 // At the end the four (m, l, O) of a row are combined through LDS with the closed form
 //   m = max m_i,  l = sum l_i 2^(m_i - m),  O = sum O_i 2^(m_i - m) / l,
 // always in the order of the waves (run-to-run bit-identical), and each output row is stored once, whole.
@@ -25,7 +26,7 @@
 // waves, twice the tile's MFMA time) and reads every byte back from LDS once, V through the transposing
 // read at half rate; and the launch has only n_kv_heads * rows / 32 workgroups (128 on a sliding layer).
 // Measured at head_dim 256: 7 us fixed + 1.1 us per tile and wave.  It beats the split kernel up to about
-// 64 visible key tiles (a sliding layer's 40: 19.9 us against 23.4 us for kernel + merge); the host picks
+// 64 visible key tiles (a sliding layer's 40: 18.5 us against 23.4 us for kernel + merge); the host picks
 // it there (dg_attn_api.hip) and the split kernel elsewhere.
 // Softmax arithmetic (lazy reference max, exponent offset under which negligible weights become exact zeros,
 // row sum over the rounded probabilities) is that of attn_mfma.hip, without its explicit zeroing of weights
@@ -168,10 +169,10 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
   // the first one, when the range starts inside it, and the last one, when the keys end inside it): block
   // blk covers rows blk * 64 / CPR ..., lane l the 16-byte chunk l of the block, swizzled.  Worked out once;
   // the tile's base address is scalar.
-  // The loads go out in groups that share one setting of M0 (lds_dma_16_group): a quarter of a K tile (its
-  // loads are spread over the softmax in quarters), two blocks of a V tile (two go between each pair of score
-  // MFMAs); the offsets carry the group's bias.
-  constexpr int GK = NBLK >= 4 ? NBLK / 4 : 1, GV = 2;
+  // The loads go out in groups that share one setting of M0 (lds_dma_16_group): four blocks of a K tile (its
+  // loads are issued together), two blocks of a V tile (two go between a pair of score MFMAs); the offsets
+  // carry the group's bias.
+  constexpr int GK = NBLK >= 4 ? 4 : NBLK, GV = 2;
   static_assert(NBLK % GK == 0 && NBLK % GV == 0 && GK <= 4, "groups tile the blocks");
   uint32_t koff[NBLK], voff[NBLK];
 #pragma unroll
@@ -348,7 +349,7 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
     const uint32_t tile = tb + jj;
     const uint32_t t0 = tile * kBlockN;
     const bool more = jj + 1u < ntile;
-    // The scores of tile jj are in s.  The K buffer takes tile jj + 1, its loads spread over the softmax.
+    // The scores of tile jj are in s.  The K buffer takes tile jj + 1.
     const TileLoad ktl = k_load(min(tile + 1u, te - 1u));
     uint32_t ktab[NBLK];
     if (__builtin_expect(tile_is_edge(min(tile + 1u, te - 1u)), 0)) {
@@ -357,10 +358,6 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
 #pragma unroll
       for (int blk = 0; blk < NBLK; ++blk) ktab[blk] = koff[blk];
     }
-    auto k_loads = [&](auto q_c) {   // a quarter of the next K tile's loads
-      constexpr int q = decltype(q_c)::value;
-      if (more) static_for<q * NGK / 4, (q + 1) * NGK / 4>([&](auto g_c) { issue_group(IsK{}, g_c, ktl, ktab); });
-    };
 
     // ---- online softmax with a lazily raised reference max ----
     if (__builtin_expect(!(t0 >= lo_max && t0 + kBlockN <= hi_min), 0)) {   // edge tile: mask
@@ -377,7 +374,10 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
       const float a4 = fmaxf(fmaxf(s[12], s[13]), s[14]);
       tmax = fmaxf(fmaxf(fmaxf(a0, a1), a2), fmaxf(fmaxf(a3, a4), s[15]));
     }
-    k_loads(std::integral_constant<int, 0>{});
+    // The scores of this tile are read (the K buffer was free since they existed): the next K tile's loads, all of
+    // them here, behind the tile max and ahead of everything that depends on it.  (Spread through the softmax
+    // in quarters they cost 0.3 us more per sliding layer, at the very top of the loop 0.1.)
+    if (more) static_for<0, NGK>([&](auto g_c) { issue_group(IsK{}, g_c, ktl, ktab); });
     tmax = max_across_halves(tmax) * p.scale_log2;
     const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kWsTau<F16>) != 0ull;
     m_run = fmaxf(m_run, tmax);
@@ -415,7 +415,6 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
       for (int i = 0; i < 4; ++i) ex[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[4 * q + i], p.scale_log2, -m_use));
       pk[q >> 1][(2 * q) & 3] = pack2<F16>(ex[0], ex[1]);
       pk[q >> 1][(2 * q + 1) & 3] = pack2<F16>(ex[2], ex[3]);
-      if constexpr (q < 3) k_loads(std::integral_constant<int, q + 1>{});
     });
     // the row sum uses the rounded probabilities, the same numbers P.V multiplies
 #pragma unroll
@@ -437,7 +436,7 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the V buffer is free for the next tile's loads
     if (more) {
       // ---- scores of tile jj + 1 (K(jj+1), the only load outstanding, has landed), with the loads of
-      // V(jj+1) between the first MFMAs: they have the rest of the scores and the softmax to land ----
+      // V(jj+1) between its MFMAs: they have the rest of the scores and the softmax to land ----
       wait_vmem_all();
       const TileLoad vtl = v_load(tile + 1u);
       uint32_t vtab[NBLK];
@@ -449,7 +448,9 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
       }
       scores([&](auto st_c) {
         constexpr int st = decltype(st_c)::value;
-        if constexpr (st < NGV) issue_group(IsV{}, st_c, vtl, vtab);
+        constexpr int first = (NSTEP - NGV) / 2;   // behind the middle MFMAs (behind the first ones: +0.15 us per
+                                                   // sliding layer, behind the last ones +0.1, after them all +0.8)
+        if constexpr (st >= first && st < first + NGV) issue_group(IsV{}, std::integral_constant<int, st - first>{}, vtl, vtab);
       });
     }
   }
