@@ -351,13 +351,7 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
     const bool more = jj + 1u < ntile;
     // The scores of tile jj are in s.  The K buffer takes tile jj + 1.
     const TileLoad ktl = k_load(min(tile + 1u, te - 1u));
-    uint32_t ktab[NBLK];
-    if (__builtin_expect(tile_is_edge(min(tile + 1u, te - 1u)), 0)) {
-      edge_table(IsK{}, ktl, ktab);
-    } else {
-#pragma unroll
-      for (int blk = 0; blk < NBLK; ++blk) ktab[blk] = koff[blk];
-    }
+    const bool k_edge = tile_is_edge(min(tile + 1u, te - 1u));
 
     // ---- online softmax with a lazily raised reference max ----
     if (__builtin_expect(!(t0 >= lo_max && t0 + kBlockN <= hi_min), 0)) {   // edge tile: mask
@@ -377,7 +371,15 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
     // The scores of this tile are read (the K buffer was free since they existed): the next K tile's loads, all of
     // them here, behind the tile max and ahead of everything that depends on it.  (Spread through the softmax
     // in quarters they cost 0.3 us more per sliding layer, at the very top of the loop 0.1.)
-    if (more) static_for<0, NGK>([&](auto g_c) { issue_group(IsK{}, g_c, ktl, ktab); });
+    if (more) {
+      if (__builtin_expect(k_edge, 0)) {   // (its own copy of the loads: the common path reads the table as it stands)
+        uint32_t etab[NBLK];
+        edge_table(IsK{}, ktl, etab);
+        static_for<0, NGK>([&](auto g_c) { issue_group(IsK{}, g_c, ktl, etab); });
+      } else {
+        static_for<0, NGK>([&](auto g_c) { issue_group(IsK{}, g_c, ktl, koff); });
+      }
+    }
     tmax = max_across_halves(tmax) * p.scale_log2;
     const bool raise = __builtin_amdgcn_ballot_w64(tmax > m_ref + kWsTau<F16>) != 0ull;
     m_run = fmaxf(m_run, tmax);
