@@ -26,7 +26,7 @@
 // waves, twice the tile's MFMA time) and reads every byte back from LDS once, V through the transposing
 // read at half rate; and the launch has only n_kv_heads * rows / 32 workgroups (128 on a sliding layer).
 // Measured at head_dim 256: 7 us fixed + 1.1 us per tile and wave.  It beats the split kernel up to about
-// 64 visible key tiles (a sliding layer's 40: 18.5 us against 23.4 us for kernel + merge); the host picks
+// 64 visible key tiles (a sliding layer's 40: 18.1 us against 23.4 us for kernel + merge); the host picks
 // it there (dg_attn_api.hip) and the split kernel elsewhere.
 // Softmax arithmetic (lazy reference max, exponent offset under which negligible weights become exact zeros,
 // row sum over the rounded probabilities) is that of attn_mfma.hip, without its explicit zeroing of weights
