@@ -582,15 +582,21 @@ __global__ void __launch_bounds__(256) attn_mfma_kernel(const AttnParams p_in) {
 #pragma unroll
           for (int i = 0; i < NDBW; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; e += 4) {
+            for (int e = 0; e < 16; e += 8) {
               f32x16& a = o[i * NRBW + j];
               float x0 = a[e], x1 = a[e + 1], x2 = a[e + 2], x3 = a[e + 3];
-              scale_acc4(x0, x1, x2, x3, corr);
+              float x4 = a[e + 4], x5 = a[e + 5], x6 = a[e + 6], x7 = a[e + 7];
+              scale_acc8(x0, x1, x2, x3, x4, x5, x6, x7, corr);
               a[e] = x0;
               a[e + 1] = x1;
               a[e + 2] = x2;
               a[e + 3] = x3;
+              a[e + 4] = x4;
+              a[e + 5] = x5;
+              a[e + 6] = x6;
+              a[e + 7] = x7;
             }
+          scale_acc_done();
         }
       }
       // O^T += V^T . P^T: per k-step, NDBW V^T fragments x NRBW P fragments.  The P fragments

@@ -44,6 +44,16 @@ template <bool F16>
 constexpr float kWsTau = F16 ? 15.9f : 120.0f;   // as attn_mfma.hip: how far a tile max may exceed the reference
 template <bool F16>
 constexpr float kWsPOff = F16 ? 0.0f : 86.0f;    // probabilities are stored as 2^(score - reference - offset)
+// With f16 probabilities a raise puts the reference this many binades ABOVE the running max, so that the next
+// raise needs a score 2^(15.9 + 4) over it: a wave of a sliding layer rescales O 3.3 times in its 10 tiles instead
+// of 5.6 (a rescale is 128 accumulation registers read, multiplied and written: as long as a tile).  The price is
+// f16's tail: a weight more than 2^(24 - 4) below the row's largest is stored with an absolute error of up to
+// 2^-25 of the reference or dropped, i.e. up to 2^-21 of the largest weight per key; this kernel sees at most 2048
+// keys per row (64 tiles, dg_attn_api.hip), so at most 2^-10 of a row's mass moves: under the rounding of a 16-bit
+// output (tests/test_gpu_parity.py builds the worst case).  The kernel for long key ranges (attn_mfma.hip) keeps a
+// reference that never leads: at 33 024 keys the same bound would be 2^-6.
+template <bool F16>
+constexpr float kWsLead = F16 ? 4.0f : 0.0f;
 
 typedef __bf16 ws_bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 ws_f16x2 __attribute__((ext_vector_type(2)));
@@ -386,7 +396,7 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
     if (__builtin_expect(raise, 0)) {
       // one row has to raise its reference: every row moves up to its running max (the block is rescaled
       // anyway, and the next raise is then as far away as it can be)
-      const float m_new = fmaxf(m_ref, m_run);
+      const float m_new = fmaxf(m_ref, m_run + kWsLead<F16>);
       const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
       const bool rescale = __builtin_amdgcn_ballot_w64(m_ref != -INFINITY && corr != 1.f) != 0ull;
       l_part *= corr;
@@ -395,14 +405,20 @@ __global__ void __launch_bounds__(256) attn_wsplit_kernel(const AttnParams p_in)
 #pragma unroll
         for (int i = 0; i < NDB; ++i)
 #pragma unroll
-          for (int e = 0; e < 16; e += 4) {
+          for (int e = 0; e < 16; e += 8) {
             float x0 = o[i][e], x1 = o[i][e + 1], x2 = o[i][e + 2], x3 = o[i][e + 3];
-            scale_acc4(x0, x1, x2, x3, corr);
+            float x4 = o[i][e + 4], x5 = o[i][e + 5], x6 = o[i][e + 6], x7 = o[i][e + 7];
+            scale_acc8(x0, x1, x2, x3, x4, x5, x6, x7, corr);
             o[i][e] = x0;
             o[i][e + 1] = x1;
             o[i][e + 2] = x2;
             o[i][e + 3] = x3;
+            o[i][e + 4] = x4;
+            o[i][e + 5] = x5;
+            o[i][e + 6] = x6;
+            o[i][e + 7] = x7;
           }
+        scale_acc_done();
       }
       m_ref = m_new;
     }

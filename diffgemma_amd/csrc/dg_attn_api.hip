@@ -24,6 +24,7 @@ constexpr size_t kAlign = 256;
 #define DG_WSPLIT_MAX_TILES 64
 #endif
 constexpr uint32_t kWsplitMaxTiles = DG_WSPLIT_MAX_TILES;
+static_assert(kWsplitMaxTiles <= 64, "attn_wsplit.hip's leading reference for f16 probabilities is sized for at most 2048 keys per row");
 
 inline size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
 inline uint32_t elem_size(uint32_t dt) { return dt == DG_F32 ? 4u : 2u; }

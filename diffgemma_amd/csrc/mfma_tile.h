@@ -74,17 +74,25 @@ __device__ __forceinline__ void mfma_scores_last(f32x16& s, u32x4 a, u32x4 b) {
 }
 
 // x *= c for values that live in accumulation registers, without the register allocator moving
-// them into the VGPR class.  Four at a time, so that no instruction waits for the one before it.
-__device__ __forceinline__ void scale_acc4(float& x0, float& x1, float& x2, float& x3, float c) {
-  float t0, t1, t2, t3;
+// them into the VGPR class.  Eight at a time: eight independent read / multiply / write chains in flight.
+__device__ __forceinline__ void scale_acc8(float& x0, float& x1, float& x2, float& x3, float& x4, float& x5, float& x6,
+                                           float& x7, float c) {
+  float t0, t1, t2, t3, t4, t5, t6, t7;
   asm volatile(
-      "v_accvgpr_read_b32 %4, %0\n\tv_accvgpr_read_b32 %5, %1\n\tv_accvgpr_read_b32 %6, %2\n\tv_accvgpr_read_b32 %7, %3\n\t"
-      "v_mul_f32 %4, %4, %8\n\tv_mul_f32 %5, %5, %8\n\tv_mul_f32 %6, %6, %8\n\tv_mul_f32 %7, %7, %8\n\t"
-      "v_accvgpr_write_b32 %0, %4\n\tv_accvgpr_write_b32 %1, %5\n\tv_accvgpr_write_b32 %2, %6\n\tv_accvgpr_write_b32 %3, %7\n\t"
-      "s_nop 3"   // the compiler does not see these writes: keep a following MFMA clear of them
-      : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+      "v_accvgpr_read_b32 %8, %0\n\tv_accvgpr_read_b32 %9, %1\n\tv_accvgpr_read_b32 %10, %2\n\tv_accvgpr_read_b32 %11, %3\n\t"
+      "v_accvgpr_read_b32 %12, %4\n\tv_accvgpr_read_b32 %13, %5\n\tv_accvgpr_read_b32 %14, %6\n\tv_accvgpr_read_b32 %15, %7\n\t"
+      "v_mul_f32 %8, %8, %16\n\tv_mul_f32 %9, %9, %16\n\tv_mul_f32 %10, %10, %16\n\tv_mul_f32 %11, %11, %16\n\t"
+      "v_mul_f32 %12, %12, %16\n\tv_mul_f32 %13, %13, %16\n\tv_mul_f32 %14, %14, %16\n\tv_mul_f32 %15, %15, %16\n\t"
+      "v_accvgpr_write_b32 %0, %8\n\tv_accvgpr_write_b32 %1, %9\n\tv_accvgpr_write_b32 %2, %10\n\tv_accvgpr_write_b32 %3, %11\n\t"
+      "v_accvgpr_write_b32 %4, %12\n\tv_accvgpr_write_b32 %5, %13\n\tv_accvgpr_write_b32 %6, %14\n\tv_accvgpr_write_b32 %7, %15"
+      : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3), "+a"(x4), "+a"(x5), "+a"(x6), "+a"(x7), "=&v"(t0), "=&v"(t1), "=&v"(t2),
+        "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7)
       : "v"(c));
 }
+// Behind the last scale_acc8 of a rescale: the compiler does not see those writes, and an MFMA that accumulates into
+// the registers must keep clear of them.  Once per rescale, not once per group of registers (a rescale of a 32-row block
+// is 16 groups at head_dim 256, and with an f16 cache a sliding layer's wave rescales every third tile).
+__device__ __forceinline__ void scale_acc_done() { asm volatile("s_nop 3"); }
 // Four values out of accumulation registers.  Spelled out so that the epilogue takes O from where
 // the tile loop left it, a few registers at a time: left to itself the compiler moves all of O
 // into VGPRs at the loop's exit, runs out of them and parks part of O in scratch memory, and the

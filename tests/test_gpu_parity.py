@@ -412,6 +412,45 @@ def test_dropped_weights_stay_below_rounding(gpu_ready, po):
         assert np.max(np.abs(lse.cpu().numpy().reshape(ref_lse.shape) - ref_lse)) < 4e-3, splits
 
 
+def test_f16_leading_reference_stays_inside_its_bound(gpu_ready, po):
+    """With an f16 cache the one-launch kernel lets its reference lead the running max by 2^4, so a weight more
+    than 2^20 below the row's largest is dropped or loses precision: at most 2^-21 of the largest weight per key,
+    2^-10 of the row's mass over the 2048 keys that kernel can see.  Rows built to make the most of it: the
+    largest key first in every wave's quarter of the keys (so that the reference is as high as it gets from the
+    start), every other key 2^21.5 below it (all dropped), as many keys as the kernel takes.  The output stays
+    inside the tolerances, and off the oracle by no more than the bound says."""
+    import torch
+    w = W.Workload("lead", 32, 2, 1, 64, 2048 - 32, rms_norm=False, seed=9, kv_f16=True)
+    assert capi.resolved_splits(w.desc()) == 1 and capi.workspace_bytes(w.desc()) == 0      # the one-launch kernel
+    q, kv = W.generate(w)
+    u = np.zeros(w.head_dim, dtype=np.float32)
+    u[:4] = 0.5                                                   # |u|^2 = 1, exact in bf16 and f16
+    q[:] = u
+    ln2 = np.float32(np.log(2.0))
+    alpha = np.full(w.t_all, (10.0 - 21.5) * ln2, dtype=np.float32)
+    alpha[[0, 512, 1024, 1536]] = 10.0 * ln2
+    alpha = R.f16_bits_to_f32(R.f32_to_f16_bits_rne(alpha))
+    kv[0] = alpha[None, :, None] * u[None, None, :]               # score of key t = alpha[t] for every row and head
+    kv[0] = R.f16_bits_to_f32(R.f32_to_f16_bits_rne(kv[0])).reshape(kv[0].shape)
+    kv[1] = R.f16_bits_to_f32(R.f32_to_f16_bits_rne(kv[1])).reshape(kv[1].shape)
+    qd, kd = W.device_arrays(w, q, kv)
+    desc = w.desc()
+    desc.out_dtype = capi.DG_F32
+    out = torch.zeros(w.canvas * w.n_q_heads * w.head_dim, dtype=torch.float32, device="cuda")
+    lse = torch.zeros(w.canvas * w.n_q_heads, dtype=torch.float32, device="cuda")
+    A.forward(desc, qd, kd, out, lse, A.alloc_workspace(desc))
+    torch.cuda.synchronize()
+    od = po.make_desc(w.canvas, w.n_q_heads, w.n_kv_heads, w.head_dim, w.kv_len, layout=w.layout, t_cap=w.t_all)
+    ref, ref_lse = po.attention_f32(od, q, kv)
+    got = out.cpu().numpy().reshape(ref.shape)
+    dropped = (w.t_all - 4) * 2.0 ** -21.5 / 4.0                  # the mass of the small keys against the four large ones
+    assert 5e-5 < dropped < 2.0 ** -10
+    vmax = float(np.abs(kv[1]).max())
+    assert max_abs_diff(got, ref) <= 2.0 * dropped * vmax + 2e-3  # what was dropped, and the f16 rounding of the kept weights
+    assert max_abs_diff(got, ref) <= MAX_ABS and mean_abs_diff(got, ref) <= MEAN_ABS
+    assert np.max(np.abs(lse.cpu().numpy().reshape(ref_lse.shape) - ref_lse)) <= dropped + 2.0 ** -11 + 1e-6
+
+
 @pytest.mark.parametrize("hd,hq,hkv", [(128, 8, 4), (512, 16, 2)])
 def test_wide_score_range_raises_reference(gpu_ready, po, hd, hq, hkv):
     """Scores that spread over hundreds of log2 units: a row's maximum climbs by more than the 2^120 the
