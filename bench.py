@@ -541,6 +541,20 @@ def other_configs():
     fl = capi.visible_pairs(desc)[1]
     recs["cfg2_sliding"] = {"ms_per_step": ms, "tflops": fl / (ms * 1e-3) / 1e12, "frac": fl / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                             "flops_per_step": fl, "launches_per_step": 1 if capi.resolved_splits(desc) == 1 else 2, "check": chk}
+    # ... and the same layer over an f16 cache, the reference's own storage (what dg_attention_dispatch runs on 25 of
+    # the model's 30 layers): f16 probabilities may lag their row's maximum by 2^15.9 only, so O is rescaled every
+    # few tiles
+    from dataclasses import replace
+    w = replace(w, name="cfg2_sliding_f16kv", kv_f16=True)
+    q, kv = W.generate(w)
+    qd, kd = W.device_arrays(w, q, kv)
+    desc = w.desc()
+    A.forward(desc, qd, kd, out, lse, ws)
+    torch.cuda.synchronize()
+    chk = oracle_rows(w, q, kv, out, lse, np.array([0, 100, 255], dtype=np.uint32))
+    ms = _graph_time(lambda: A.forward(desc, qd, kd, out, lse, ws), 100, 5)
+    recs["cfg2_sliding_f16kv"] = {"ms_per_step": ms, "tflops": fl / (ms * 1e-3) / 1e12, "frac": fl / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                  "flops_per_step": fl, "launches_per_step": 1 if capi.resolved_splits(desc) == 1 else 2, "check": chk}
 
     # ---- configuration 4: 131072-key prefix, 1 % of the prefix keys scaled x8 (generated on the device: the host
     # generator of the parity tests takes longer than this whole pass may) ----
